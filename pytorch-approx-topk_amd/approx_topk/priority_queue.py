@@ -1,0 +1,104 @@
+"""``approx_topk.topk``: bucketed approximate top-k on AMD GPUs.
+
+Same operator name, signature, defaults and error behaviour as the reference's
+approx_topk/priority_queue.py:14-110; the body calls hand-written HIP kernels
+through the C ABI of libapprox_topk_hip.so instead of a JIT-built CUDA module.
+"""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from . import _native
+
+
+def _result_shape(xs: Tensor, k: int, dim: int) -> list[int]:
+    shape = list(xs.shape)
+    shape[dim] = k
+    return shape
+
+
+def _empty_result(xs: Tensor, k: int, dim: int) -> tuple[Tensor, Tensor]:
+    shape = _result_shape(xs, k, dim)
+    return (torch.empty(shape, dtype=xs.dtype, device=xs.device),
+            torch.empty(shape, dtype=torch.int64, device=xs.device))
+
+
+@torch.library.custom_op("approx_topk::topk", mutates_args=())
+def topk(
+    xs: Tensor,
+    k: int,
+    dim: int,
+    j: int = 1,
+    k_mult: int = 1,
+    interleaved: bool = True,
+    multithread_buckets: bool | None = False,
+) -> tuple[Tensor, Tensor]:
+    """Approximate top-``k`` of ``xs`` along ``dim``.
+
+    The slice is cut into ``b = k_mult * k / j`` buckets (interleaved: bucket
+    ``c`` holds positions ``c, c+b, c+2b, ...``; otherwise contiguous runs), the
+    ``j`` largest of every bucket are kept, and if that leaves more than ``k``
+    candidates (``k_mult > 1``) an exact top-``k`` of the candidates follows.
+
+    Returns ``(values, indices)`` shaped like ``xs`` with ``dim`` of size ``k``;
+    ``values`` has the dtype of ``xs``, ``indices`` is int64, and
+    ``xs.gather(dim, indices) == values``.  The order along ``dim`` is
+    deterministic but carries no meaning.  Ties between equal values go to the
+    lowest index.
+
+    :param j: elements kept per bucket, 1..4; must divide ``k * k_mult``.
+    :param k_mult: factor on the number of stage-1 candidates; >= 1.
+    :param multithread_buckets: accepted for compatibility; the kernels choose
+        their own work split from the shape.
+    """
+    if dim < 0:
+        dim += xs.ndim
+    last = xs.ndim - 1
+    if j < k and dim != last:
+        raise NotImplementedError("This topk only currently works on the last dim")
+    if k_mult < 1:
+        raise ValueError(f"k_mult must be >=1, was {k_mult}")
+    k0 = k * k_mult
+
+    if k0 == 0:
+        return _empty_result(xs, 0, dim)
+    if j < 1 or j > 4:
+        raise RuntimeError("topk: j must 0 < j < 5")
+    if k0 % j != 0:
+        raise RuntimeError("topk: j must divide k")
+    n = xs.shape[dim] if xs.ndim else 1
+    if k0 > n:
+        raise RuntimeError("topk: k must not be larger than topk size")
+    _native.require_gpu(xs)
+    if xs.numel() == 0:
+        return _empty_result(xs, k, dim)
+
+    layout = _native.INTERLEAVED if interleaved else _native.BALANCED
+    rows = xs if xs.ndim else xs.reshape(1)
+    moved = dim != last and xs.ndim > 1
+    if moved:
+        rows = rows.movedim(dim, -1)
+    if k_mult == 1:
+        values, indices = _native.stage1(rows, k0, j, layout)
+    else:
+        values, indices = _native.topk(rows, k0, j, k, layout)
+    if moved:
+        values = values.movedim(-1, dim).contiguous()
+        indices = indices.movedim(-1, dim).contiguous()
+    if not xs.ndim:
+        values, indices = values.reshape(()), indices.reshape(())
+    return values, indices
+
+
+@topk.register_fake
+def _(
+    xs: Tensor,
+    k: int,
+    dim: int,
+    j: int | None = None,
+    k_mult: int = 1,
+    interleaved: bool = True,
+    multithread_buckets: bool | None = False,
+) -> tuple[Tensor, Tensor]:
+    return _empty_result(xs, k, dim)

@@ -1,0 +1,72 @@
+"""Builds libapprox_topk_hip.so for gfx950 with hipcc, in-tree.
+
+    python pytorch-approx-topk_amd/build.py [--force]
+
+Every .hip file under csrc/ is compiled to an object (in parallel) and linked
+into approx_topk/libapprox_topk_hip.so, next to the Python package that loads
+it.  Nothing is linked against libtorch: the library speaks a C ABI only.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "approx_topk", "libapprox_topk_hip.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra",
+    # Packed FP32 instructions are kept out of the device code on purpose.
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _newer(target: str, deps: list[str]) -> bool:
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(d) <= t for d in deps)
+
+
+def build(force: bool = False, verbose: bool = True) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    headers = sorted(glob.glob(os.path.join(CSRC, "*.h"))) + [
+        os.path.join(os.path.dirname(HERE), "include", "approx_topk_hip.h")]
+    jobs = []
+    objects = []
+    for src in sources:
+        obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+        objects.append(obj)
+        if force or not _newer(obj, [src] + headers):
+            jobs.append([HIPCC, *FLAGS, "-c", src, "-o", obj])
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        return cmd, r
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
+        for cmd, r in ex.map(run, jobs):
+            # hipcc's host pass warns that it does not know the packed-fp32 feature.
+            err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+            if r.returncode != 0:
+                raise RuntimeError(f"{' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
+            if verbose and err.strip():
+                print(err, file=sys.stderr)
+    if force or jobs or not _newer(LIB, objects):
+        cmd, r = run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objects])
+        if r.returncode != 0:
+            raise RuntimeError(f"{' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv))

@@ -1,0 +1,118 @@
+// extern "C" entry points of libapprox_topk_hip.so: argument checks and the
+// choice of kernel.  Everything here runs on the host and only enqueues work.
+#include "atk_device.h"
+#include "atk_launch.h"
+
+namespace {
+
+constexpr int kAbiVersion = 1;
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+int check_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0,
+                 int j, int layout, int dtype, const void* values, const void* indices) {
+  if (atk::elem_bytes(dtype) == 0) return ATK_ERR_DTYPE;
+  if (layout < ATK_INTERLEAVED || layout > ATK_INTERLEAVED_PADDED) return ATK_ERR_LAYOUT;
+  if (rows < 0 || n < 0 || k0 < 0) return ATK_ERR_K;
+  if (k0 == 0 || rows == 0) return ATK_OK;
+  if (j < 1 || j > 4 || k0 % j) return ATK_ERR_J;
+  const bool padded = layout == ATK_CEIL_CHUNK || layout == ATK_INTERLEAVED_PADDED;
+  if (padded && j != 1) return ATK_ERR_LAYOUT;
+  if (padded ? n < 1 : k0 > n) return ATK_ERR_K;
+  if (!x || !values || !indices || row_stride < n) return ATK_ERR_ARG;
+  return ATK_OK;
+}
+
+struct TopkPlan {
+  size_t cand_values_off, cand_indices_off, total;
+};
+
+TopkPlan plan_topk(int64_t rows, int64_t k0, int64_t k, int dtype) {
+  TopkPlan p{0, 0, 0};
+  if (k == k0 || rows <= 0 || k0 <= 0) return p;
+  const size_t vals = align_up((size_t)rows * (size_t)k0 * atk::elem_bytes(dtype), 256);
+  p.cand_values_off = 0;
+  p.cand_indices_off = vals;
+  p.total = vals + align_up((size_t)rows * (size_t)k0 * sizeof(int64_t), 256);
+  return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+int atk_version(void) { return kAbiVersion; }
+
+const char* atk_strerror(int status) {
+  switch (status) {
+    case ATK_OK: return "ok";
+    case ATK_ERR_DTYPE: return "unsupported element type";
+    case ATK_ERR_J: return "topk: j must satisfy 0 < j < 5 and j must divide k";
+    case ATK_ERR_K: return "topk: k must not be larger than topk size";
+    case ATK_ERR_LAYOUT: return "unknown bucket layout, or a padded layout with j != 1";
+    case ATK_ERR_WORKSPACE: return "workspace missing or too small";
+    case ATK_ERR_LAUNCH: return "HIP kernel launch failed";
+    case ATK_ERR_ARG: return "invalid pointer or stride argument";
+    case ATK_ERR_TOO_LARGE: return "topk: too many buckets or slices";
+  }
+  return "unknown status";
+}
+
+size_t atk_stage1_workspace_bytes(int64_t, int64_t, int64_t, int, int, int) { return 0; }
+
+int atk_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+               int layout, int dtype, void* values, int64_t* indices, void* ws,
+               size_t ws_bytes, atk_stream_t stream) {
+  (void)ws; (void)ws_bytes;
+  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices);
+  if (rc != ATK_OK || k0 == 0 || rows == 0) return rc;
+  return atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout, dtype,
+                                            values, indices, (hipStream_t)stream);
+}
+
+size_t atk_select_workspace_bytes(int64_t, int64_t, int64_t, int) { return 0; }
+
+int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
+               int64_t k, int64_t index_bound, int dtype, void* values, int64_t* indices,
+               void* ws, size_t ws_bytes, atk_stream_t stream) {
+  (void)ws; (void)ws_bytes;
+  if (atk::elem_bytes(dtype) == 0) return ATK_ERR_DTYPE;
+  if (rows < 0 || k0 < 0 || k < 0 || k > k0 || index_bound < 0) return ATK_ERR_K;
+  if (rows == 0 || k == 0) return ATK_OK;
+  if (!cand_values || !cand_indices || !values || !indices) return ATK_ERR_ARG;
+  return atk::launch_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype,
+                            values, indices, (hipStream_t)stream);
+}
+
+size_t atk_topk_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int64_t k,
+                                int layout, int dtype) {
+  (void)n; (void)j; (void)layout;
+  return plan_topk(rows, k0, k, dtype).total;
+}
+
+int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+             int64_t k, int layout, int dtype, void* values, int64_t* indices, void* ws,
+             size_t ws_bytes, atk_stream_t stream) {
+  if (k < 0 || k > k0) return ATK_ERR_K;
+  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices);
+  if (rc != ATK_OK || k == 0 || rows == 0) return rc;
+  if (k == k0)
+    return atk_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws,
+                      ws_bytes, stream);
+  const TopkPlan p = plan_topk(rows, k0, k, dtype);
+  if (!ws || ws_bytes < p.total) return ATK_ERR_WORKSPACE;
+  unsigned char* base = static_cast<unsigned char*>(ws);
+  void* cand_values = base + p.cand_values_off;
+  int64_t* cand_indices = reinterpret_cast<int64_t*>(base + p.cand_indices_off);
+  const int rc1 = atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout,
+                                                     dtype, cand_values, cand_indices,
+                                                     (hipStream_t)stream);
+  if (rc1 != ATK_OK) return rc1;
+  const int64_t bound = (layout == ATK_CEIL_CHUNK || layout == ATK_INTERLEAVED_PADDED)
+                            ? ((n + k0 - 1) / k0) * k0
+                            : n;
+  return atk::launch_select(cand_values, cand_indices, rows, k0, k, bound, dtype, values,
+                            indices, (hipStream_t)stream);
+}
+
+}  // extern "C"

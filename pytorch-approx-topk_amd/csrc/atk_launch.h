@@ -1,0 +1,22 @@
+// Host-side launchers shared between the translation units of the library.
+// Each returns an atk_status and only enqueues work on `stream`.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace atk {
+
+// stage1_lane_per_bucket.hip: any dtype / layout / shape.
+int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
+                                  int64_t row_stride, int64_t k0, int j, int layout,
+                                  int dtype, void* values, int64_t* indices,
+                                  hipStream_t stream);
+
+// stage2_radix_select.hip: one workgroup per row.
+int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
+                  int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
+                  int64_t* indices, hipStream_t stream);
+
+}  // namespace atk

@@ -1,0 +1,252 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the
+same seeded inputs -- values bit-exact, indices identical, same output order.
+Shapes follow the reference's own tests (tests/test_priority_queue.py)."""
+import pytest
+import torch
+
+import oracle
+from helpers import assert_same, cpu_randn, oracle_topk
+
+pytestmark = pytest.mark.gpu
+
+FLOATS = [torch.float32, torch.bfloat16, torch.float16]
+ALL_DTYPES = FLOATS + [torch.float64, torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64]
+
+
+def _topk():
+    from approx_topk import topk
+    return topk
+
+
+def _run(x_cpu, k, dim=-1, **kw):
+    v, i = _topk()(x_cpu.cuda(), k, dim, **kw)
+    torch.cuda.synchronize()
+    return v, i
+
+
+def _check(x_cpu, k, dim=-1, what="", **kw):
+    v, i = _run(x_cpu, k, dim, **kw)
+    kw.pop("multithread_buckets", None)
+    ev, ei = oracle_topk(x_cpu, k, dim, **kw)
+    assert_same(v, i, ev, ei, what or f"shape={tuple(x_cpu.shape)} k={k} dim={dim} {kw}")
+    if k:
+        assert torch.equal(x_cpu.gather(dim, i.cpu()).view(torch.uint8 if x_cpu.element_size() == 1 else
+                                                           {2: torch.int16, 4: torch.int32, 8: torch.int64}[x_cpu.element_size()]),
+                           v.cpu().view(torch.uint8 if x_cpu.element_size() == 1 else
+                                        {2: torch.int16, 4: torch.int32, 8: torch.int64}[x_cpu.element_size()]))
+
+
+@pytest.mark.parametrize("k", [0, 2, 4])
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("multithread_buckets", [False, True])
+def test_one_bucket_no_batch_equals_exact(k, dtype, interleaved, multithread_buckets):
+    x = cpu_randn(1001, 234, dtype)
+    v, i = _run(x, k, 0, j=k, interleaved=interleaved, multithread_buckets=multithread_buckets)
+    ev, ei = torch.topk(x.float(), k, dim=0)
+    assert torch.equal(v.cpu().float().sort().values, ev.sort().values)
+    assert torch.equal(x[i.cpu()], v.cpu())
+    if k:
+        _check(x, k, 0, j=k, interleaved=interleaved)
+
+
+@pytest.mark.parametrize("k", [0, 2, 4])
+@pytest.mark.parametrize("dim", [0, 1, 2])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_one_bucket_batched_any_dim(k, dim, interleaved):
+    g = torch.Generator().manual_seed(4242)
+    x = torch.rand((30, 25, 16), generator=g)
+    v, i = _run(x, k, dim, j=k, interleaved=interleaved)
+    ev, ei = torch.topk(x, k, dim)
+    assert torch.equal(v.cpu().sort(dim).values, ev.sort(dim).values)
+    assert torch.equal(i.cpu().sort(dim).values, ei.sort(dim).values)
+    assert v.is_contiguous() and list(v.shape) == list(ev.shape)
+
+
+@pytest.mark.parametrize("dim", [-1, -2])
+def test_negative_dim(dim):
+    x = cpu_randn((128, 256), 99)
+    _check(x, 4, dim, j=4)
+
+
+def test_call_twice_same_result():
+    x = cpu_randn((128,), 56)
+    a = _run(x, 4, 0)
+    b = _run(x, 4, 0)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+@pytest.mark.parametrize("n", [10, 16])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_bucket_size_one_no_batch(n, interleaved):
+    x = cpu_randn(n, 856)
+    v, i = _run(x, n, 0, j=1, interleaved=interleaved)
+    assert torch.equal(i.cpu(), torch.arange(n)) and torch.equal(v.cpu(), x)
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_bucket_size_one_batched(dtype, interleaved):
+    x = cpu_randn((16, 4, 12), 23, dtype)
+    v, i = _run(x, 12, 2, j=1, interleaved=interleaved)
+    ev, ei = torch.topk(x.float(), 12, 2)
+    assert torch.equal(v.cpu().float().sort(2).values, ev.sort(2).values)
+    _check(x, 12, 2, j=1, interleaved=interleaved)
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_k_mult_bucket_size_one_equals_exact(dtype, interleaved):
+    # 1024 buckets of one element, then an exact top-64 of all of them
+    x = cpu_randn((32, 1024), 23, dtype)
+    v, i = _run(x, 64, -1, k_mult=16, j=1, interleaved=interleaved)
+    ev, ei = torch.topk(x.float(), 64, -1)
+    assert torch.equal(v.cpu().float().sort(-1).values, ev.sort(-1).values)
+    _check(x, 64, -1, k_mult=16, j=1, interleaved=interleaved)
+
+
+def _ideal_rows(n, hot):
+    xs = torch.zeros(len(hot), n)
+    for r, cells in enumerate(hot):
+        for pos, val in cells:
+            xs[r, pos] = val
+    return xs
+
+
+def test_ideal_contiguous_n17():
+    x = _ideal_rows(17, [
+        [(0, 11.), (4, 12.), (5, 13.), (8, 14.), (9, 15.), (12, 16.), (13, 17.), (16, 18.)],
+        [(2, 21.), (3, 22.), (6, 23.), (7, 24.), (10, 25.), (11, 26.), (14, 27.), (15, 28.)]])
+    v, i = _run(x, 8, 1, j=2, interleaved=False)
+    ev, ei = torch.topk(x, 8, dim=1)
+    assert torch.equal(v.cpu().sort(1).values, ev.sort(1).values)
+    assert torch.equal(i.cpu().sort(1).values, ei.sort(1).values)
+
+
+def test_ideal_interleaved_n17():
+    x = _ideal_rows(17, [
+        [(0, 11.), (16, 12.), (1, 13.), (13, 14.), (2, 15.), (14, 16.), (3, 17.), (15, 18.)],
+        [(4, 21.), (8, 22.), (5, 23.), (9, 24.), (6, 25.), (10, 26.), (7, 27.), (11, 28.)]])
+    v, i = _run(x, 8, 1, j=2, interleaved=True)
+    ev, ei = torch.topk(x, 8, dim=1)
+    assert torch.equal(v.cpu().sort(1).values, ev.sort(1).values)
+    assert torch.equal(i.cpu().sort(1).values, ei.sort(1).values)
+
+
+def test_contiguous_long_sequence_n10000():
+    n, k, j, stride = 10_000, 8, 2, 625
+    g = torch.Generator().manual_seed(1)
+    x = torch.zeros(2, n)
+    x[0, list(range(0, n, stride))] = torch.rand(n // stride, generator=g) + 2.0
+    x[1, list(range(50, n, stride))] = torch.rand(n // stride, generator=g) + 2.0
+    _check(x, k, 1, j=j, interleaved=False)
+
+
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("j", [1, 2, 4])
+@pytest.mark.parametrize("k_mult", [1, 2, 4])
+def test_reference_parity_shape(interleaved, j, k_mult):
+    # randn(5, 32, 512), k=64: the shape of the reference's kernel-vs-torch test
+    x = cpu_randn((5, 32, 512), 100)
+    _check(x, 64, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+    v, i = _run(x, 64, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+    tv, ti = oracle.torch_bucketed_topk(x, 64, j, k_mult) if interleaved else (None, None)
+    if tv is not None:
+        assert torch.equal(v.cpu().sort(-1).values, tv.sort(-1).values)
+        assert torch.equal(i.cpu().sort(-1).values, ti.sort(-1).values)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("j,k_mult", [(1, 1), (2, 2), (3, 1), (4, 4)])
+def test_all_dtypes_with_ties(dtype, interleaved, j, k_mult):
+    g = torch.Generator().manual_seed(7 + j)
+    if dtype.is_floating_point:
+        x = torch.randint(-6, 7, (3, 7, 333), generator=g).to(dtype) / 2
+    elif dtype == torch.uint8:
+        x = torch.randint(0, 12, (3, 7, 333), generator=g).to(dtype)
+    else:
+        x = torch.randint(-6, 7, (3, 7, 333), generator=g).to(dtype)
+    _check(x, 12, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+def test_special_values(dtype):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn((4, 4096), generator=g).to(dtype)
+    sel = torch.randint(0, 4096, (4, 200), generator=g)
+    specials = torch.tensor([float("nan"), float("inf"), -float("inf"), 0.0, -0.0]).to(dtype)
+    for r in range(4):
+        x[r, sel[r]] = specials[torch.randint(0, 5, (200,), generator=g)]
+    for j, km in [(1, 1), (2, 1), (4, 2), (1, 4)]:
+        _check(x, 256, -1, j=j, k_mult=km)
+        _check(x, 256, -1, j=j, k_mult=km, interleaved=False)
+
+
+@pytest.mark.parametrize("n,k,j", [(17, 8, 2), (1001, 12, 4), (1000, 16, 1), (65, 64, 1), (4099, 33, 3),
+                                   (5000, 1250, 2), (70001, 4096, 4)])
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_ragged_shapes(n, k, j, interleaved):
+    x = cpu_randn((3, n), n + k)
+    _check(x, k, -1, j=j, interleaved=interleaved)
+
+
+def test_all_equal_rows_cut_ties_by_index():
+    x = torch.zeros(2, 4096)
+    x[1] = 1.5
+    for j, km in [(1, 2), (2, 4), (4, 8)]:
+        _check(x, 128, -1, j=j, k_mult=km)
+
+
+def test_row_stride_input():
+    big = cpu_randn((6, 3000), 5)
+    xg = big.cuda()[:, :2048]
+    v, i = _topk()(xg, 64, -1, j=2, k_mult=2)
+    ev, ei = oracle_topk(big[:, :2048].contiguous(), 64, -1, j=2, k_mult=2)
+    assert_same(v, i, ev, ei, "strided rows")
+
+
+def test_config_shapes_reduced():
+    # C2-like (L=32 interleaved, no stage 2), C3-like fp16, C4-like, C5-like
+    _check(cpu_randn((4, 1 << 16), 1002), 4096, -1, j=2)
+    _check((cpu_randn((8, 32768), 1003) / 128 ** 0.5).half(), 2048, -1, j=4, k_mult=4)
+    _check(cpu_randn((4, 131072), 1004), 64, -1, j=1, k_mult=8)
+    n = 1 << 20
+    x = 0.5 * torch.linspace(-1, 1, n) + cpu_randn((n,), 1005)
+    _check(x.reshape(1, n), 1024, -1, j=4, k_mult=2)
+
+
+def test_errors_match_reference_types():
+    topk = _topk()
+    x = torch.randn(8, 64, device="cuda")
+    with pytest.raises(NotImplementedError):
+        topk(x, 4, 0, j=2)
+    with pytest.raises(ValueError):
+        topk(x, 4, -1, k_mult=0)
+    with pytest.raises(RuntimeError):
+        topk(x, 6, -1, j=4)
+    with pytest.raises(RuntimeError):
+        topk(x, 5, -1, j=5)
+    with pytest.raises(RuntimeError):
+        topk(x, 128, -1)
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("multithread_buckets", [None, False, True])
+def test_opcheck(dtype, interleaved, multithread_buckets):
+    x = cpu_randn((32, 128), 0, dtype).cuda()
+    torch.library.opcheck(_topk(), args=(x,), kwargs=dict(
+        k=12, dim=-1, j=1, interleaved=interleaved, multithread_buckets=multithread_buckets))
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_torch_compile_fullgraph(dtype, interleaved):
+    topk = _topk()
+    compiled = torch.compile(topk, fullgraph=True)
+    x = cpu_randn((32, 128), 0, dtype).cuda()
+    kw = dict(xs=x, k=12, dim=-1, j=2, interleaved=interleaved, multithread_buckets=None)
+    ev, ei = topk(**kw)
+    cv, ci = compiled(**kw)
+    assert torch.equal(ev, cv) and torch.equal(ei, ci)

@@ -1,0 +1,121 @@
+"""CPU-side checks: the C-ABI library loads and exports every declared symbol,
+argument validation raises the reference's exception types before any GPU work,
+and the torch-level entry points agree with the oracle."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from approx_topk import _native
+    header = open(os.path.join(ROOT, "include", "approx_topk_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(atk_[a-z0-9_]+)\s*\(", header))
+    assert {"atk_version", "atk_strerror", "atk_stage1", "atk_select", "atk_topk"} <= declared
+    handle = ctypes.CDLL(_native.library_path())
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert set(_native._SIGNATURES) == declared
+    assert _native.lib().atk_version() == _native.ABI_VERSION
+    assert _native.lib().atk_strerror(0) == b"ok"
+    assert b"j must" in _native.lib().atk_strerror(-2)
+
+
+def test_native_argument_checks_need_no_gpu():
+    # rejected before any launch, so callable here
+    from approx_topk import _native
+    L = _native.lib()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    assert L.atk_stage1(p, 1, 8, 8, 6, 4, 0, 0, p, p, None, 0, None) == -2     # j does not divide k0
+    assert L.atk_stage1(p, 1, 8, 8, 5, 5, 0, 0, p, p, None, 0, None) == -2     # j out of range
+    assert L.atk_stage1(p, 1, 8, 8, 16, 1, 0, 0, p, p, None, 0, None) == -3    # k0 > n
+    assert L.atk_stage1(p, 1, 8, 8, 4, 1, 9, 0, p, p, None, 0, None) == -4     # layout
+    assert L.atk_stage1(p, 1, 8, 8, 4, 2, 2, 0, p, p, None, 0, None) == -4     # padded layout, j != 1
+    assert L.atk_stage1(p, 1, 8, 8, 4, 1, 0, 99, p, p, None, 0, None) == -1    # dtype
+    assert L.atk_stage1(None, 1, 8, 8, 4, 1, 0, 0, p, p, None, 0, None) == -7  # null input
+    assert L.atk_stage1(p, 1, 8, 4, 4, 1, 0, 0, p, p, None, 0, None) == -7     # row_stride < n
+    assert L.atk_stage1(p, 1, 8, 8, 0, 1, 0, 0, p, p, None, 0, None) == 0      # k0 == 0: no-op
+    assert L.atk_topk(p, 1, 8, 8, 4, 1, 2, 0, 0, p, p, None, 0, None) == -5    # workspace missing
+    assert L.atk_topk(p, 1, 8, 8, 4, 1, 5, 0, 0, p, p, None, 0, None) == -3    # k > k0
+    assert L.atk_select(p, p, 1, 4, 5, 8, 0, p, p, None, 0, None) == -3
+    assert L.atk_topk_workspace_bytes(3, 100, 8, 1, 8, 0, 0) == 0
+    assert L.atk_topk_workspace_bytes(3, 100, 16, 1, 8, 0, 0) >= 3 * 16 * 12
+
+
+def test_validation_errors_before_device_check():
+    from approx_topk import topk
+    x = torch.randn(8, 64)
+    with pytest.raises(NotImplementedError):
+        topk(x, 4, 0, j=2)
+    with pytest.raises(ValueError):
+        topk(x, 4, -1, k_mult=0)
+    with pytest.raises(RuntimeError, match="j must divide k"):
+        topk(x, 6, -1, j=4)
+    with pytest.raises(RuntimeError, match="0 < j < 5"):
+        topk(x, 5, -1, j=5)
+    with pytest.raises(RuntimeError, match="k must not be larger"):
+        topk(x, 128, -1)
+    with pytest.raises(RuntimeError, match="GPU"):
+        topk(x, 4, -1)          # valid arguments, but no CPU path exists
+    v, i = topk(x, 0, -1, j=0)  # k == 0 is valid and does no work
+    assert v.shape == (8, 0) and i.dtype == torch.int64
+
+
+def test_fake_impl_shapes():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from approx_topk import topk
+    with FakeTensorMode():
+        x = torch.empty(5, 32, 512)
+        v, i = topk(x, 64, -1, j=2, k_mult=2)
+        assert v.shape == (5, 32, 64) and i.shape == (5, 32, 64)
+        assert v.dtype == torch.float32 and i.dtype == torch.int64
+
+
+def test_topk_torch_known_answers_and_oracle():
+    from approx_topk.experimental.bucketed_argmax import topk_torch
+    x = torch.stack([100 * torch.arange(0, 20), -100 * torch.arange(0, 20)]).float()
+    v, i = topk_torch(x, k=3, dim=1, interleaved=False)
+    assert v.tolist() == [[600.0, 1300, 1900], [0, -700, -1400]] and i.tolist() == [[6, 13, 19], [0, 7, 14]]
+    vt, it = topk_torch(x.T, k=3, dim=0, interleaved=False)
+    assert torch.equal(vt.T, v) and torch.equal(it.T, i)
+    v, i = topk_torch(x, k=3, dim=1, interleaved=True)
+    assert v.tolist() == [[1800.0, 1900, 1700], [0, -100, -200]] and i.tolist() == [[18, 19, 17], [0, 1, 2]]
+    g = torch.Generator().manual_seed(1001)
+    c1 = torch.randn(4, 65536, generator=g)
+    for interleaved in (True, False):
+        v, i = topk_torch(c1, 1024, -1, interleaved)
+        ev, ei = oracle.bucketed_argmax(c1, 1024, -1, interleaved)
+        assert torch.equal(v, ev) and torch.equal(i, ei)
+
+
+def test_batch_contiguous():
+    from approx_topk.experimental.bucketed_argmax import _batch_contiguous
+    x = torch.arange(3 * 4 * 5).view(3, 4, 5)
+    for t, same in [(x, True), (x[:, :, :-1], True), (x[:, :, ::2], False), (x[:, :-1, :], False),
+                    (x.swapdims(0, 1), False)]:
+        t2 = _batch_contiguous(t)
+        assert (t2 is t) == same
+        assert torch.equal(t, t2)
+        if not same:
+            assert t2.is_contiguous()
+
+
+def test_rows_view():
+    from approx_topk import _native
+    x = torch.arange(3 * 4 * 10.0).view(3, 4, 10)
+    t, rows, n, step = _native.rows_view(x)
+    assert t is x and (rows, n, step) == (12, 10, 10)
+    t, rows, n, step = _native.rows_view(x[:, :, :7])
+    assert t.data_ptr() == x.data_ptr() and (rows, n, step) == (12, 7, 10)
+    t, rows, n, step = _native.rows_view(x[:, :3, :])
+    assert t.is_contiguous() and (rows, n, step) == (9, 10, 10)
+    t, rows, n, step = _native.rows_view(x.movedim(1, -1))
+    assert t.is_contiguous() and (rows, n, step) == (30, 4, 4)
