@@ -96,7 +96,7 @@ __global__ __launch_bounds__(1024) void select_kernel(
   key_t prefix = 0, mask = 0;
   uint32_t need = k;
   for (int shift = E::key_bits - 8; shift >= 0; shift -= 8) {
-    if (tid < 256) sh.hist[tid] = 0;
+    for (uint32_t i = tid; i < 256; i += nt) sh.hist[i] = 0;
     __syncthreads();
     for (uint32_t i = tid; i < k0; i += nt) {
       const key_t key = key_at(i);
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(1024) void select_kernel(
     uint64_t iprefix = 0, imask = 0;
     for (int shift = ((index_bits + 7) / 8 - 1) * 8; shift >= 0; shift -= 8) {
       __syncthreads();
-      if (tid < 256) sh.hist[tid] = 0;
+      for (uint32_t i = tid; i < 256; i += nt) sh.hist[i] = 0;
       __syncthreads();
       for (uint32_t i = tid; i < k0; i += nt) {
         if (key_at(i) == T) {
