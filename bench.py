@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""Benchmark of the bucketed approximate top-k hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all-configs]
+
+A "step" is one ``approx_topk.topk`` call over one batch of synthetic input that
+already sits in HBM.  The workload is the headline shape: fp32 x[128, 2^20]
+iid N(0,1), k = 65536, j = 2, k_mult = 1 (32768 interleaved buckets of 32).
+Inputs rotate over several distinct tensors so that the working set is larger
+than the last-level cache.  One JSON line is printed on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "pytorch-approx-topk_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+# name -> (rows, n, dtype, k, j, k_mult, seed)
+CONFIGS = {
+    "C1": (4, 65536, "float32", 1024, 1, 1, 1001),
+    "C2": (128, 1 << 20, "float32", 65536, 2, 1, 1002),
+    "C3": (1024, 32768, "float16", 2048, 4, 4, 1003),
+    "C4": (256, 131072, "float32", 64, 1, 8, 1004),
+    "C5": (1, 1 << 26, "float32", 16384, 4, 2, 1005),
+}
+
+
+def make_input(name: str, variant: int = 0):
+    """Synthetic input of a config, generated on the CPU from a fixed seed."""
+    import numpy as np
+    import torch
+
+    rows, n, dtype, k, j, km, seed = CONFIGS[name]
+    g = torch.Generator().manual_seed(seed + 7919 * variant)
+    if name == "C3":
+        x = (torch.randn(rows, n, generator=g) / math.sqrt(128.0)).half()
+    elif name == "C4":
+        x = torch.randn(rows, n, generator=g)
+        rng = np.random.default_rng(seed + 7919 * variant)
+        hot = n // 100
+        for r in range(rows):
+            cols = torch.randperm(n, generator=g)[:hot]
+            x[r, cols] += torch.from_numpy(rng.zipf(1.1, hot).astype(np.float32))
+    elif name == "C5":
+        x = 0.5 * torch.linspace(-1, 1, n).reshape(1, n) + torch.randn(rows, n, generator=g)
+    else:
+        x = torch.randn(rows, n, generator=g)
+    return x
+
+
+def recall_at_k(approx_values, exact_values, k: int) -> float:
+    """mean over rows of count(approx >= k-th exact value) / k
+    (definition of benchmarks/run_recall.py:31-36 in the reference)."""
+    kth = exact_values.min(dim=-1, keepdim=True).values
+    return float(((approx_values >= kth).sum(-1).double() / k).mean())
+
+
+def time_config(name: str, steps: int, warmup: int, n_inputs: int):
+    import torch
+
+    from approx_topk import topk
+
+    rows, n, dtype, k, j, km, seed = CONFIGS[name]
+    esize = 2 if dtype == "float16" else 4
+    # enough distinct inputs to exceed a 256 MiB last-level cache
+    per = rows * n * esize
+    n_inputs = max(n_inputs, min(8, -(-(600 << 20) // per)))
+    xs = [make_input(name, v).cuda() for v in range(n_inputs)]
+    torch.cuda.synchronize()
+    for s in range(warmup):
+        topk(xs[s % n_inputs], k, -1, j=j, k_mult=km)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for s in range(steps):
+        topk(xs[s % n_inputs], k, -1, j=j, k_mult=km)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = start.elapsed_time(stop)
+    return xs, wall, dev_ms, rows * n, per
+
+
+def parity_and_recall(name: str, x_gpu, sample_rows: int):
+    """Oracle check on a few rows (bit-exact) and recall against exact torch.topk."""
+    import torch
+
+    import oracle
+    from approx_topk import topk
+
+    rows, n, dtype, k, j, km, seed = CONFIGS[name]
+    v, i = topk(x_gpu, k, -1, j=j, k_mult=km)
+    exact = torch.topk(x_gpu.float(), k, dim=-1).values
+    rec = recall_at_k(v.float(), exact, k)
+    take = min(sample_rows, rows)
+    ev, ei = oracle.topk(x_gpu[:take].cpu(), k, -1, j=j, k_mult=km)
+    bits = torch.int16 if dtype == "float16" else torch.int32
+    ok = bool(torch.equal(v[:take].cpu().view(bits), ev.view(bits)) and torch.equal(i[:take].cpu(), ei))
+    return rec, ok, take
+
+
+def cpu_baseline(name: str):
+    """Torch-level bucketed top-k (the reference's CPU-capable algorithm, restated
+    in oracle/) timed on this machine's host cores over the full workload."""
+    import torch
+
+    import oracle
+
+    rows, n, dtype, k, j, km, seed = CONFIGS[name]
+    x = make_input(name)
+    oracle.torch_bucketed_topk(x, k, j, km)  # warm-up
+    times = []
+    for _ in range(3):
+        t = time.perf_counter()
+        oracle.torch_bucketed_topk(x, k, j, km)
+        times.append(time.perf_counter() - t)
+    med = sorted(times)[1]
+    esize = x.element_size()
+    return {
+        "value": rows * n * esize / med / 1e9,
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"all {rows} rows of the workload, median of 3 runs after 1 warm-up "
+                  f"({med:.3f} s per pass, {rows * n / med / 1e9:.3f} G elem/s, os.cpu_count()={os.cpu_count()})",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--inputs", type=int, default=5, help="distinct input tensors to rotate over")
+    ap.add_argument("--workload", default="C2", choices=sorted(CONFIGS))
+    ap.add_argument("--all-configs", action="store_true", help="also time C3, C4, C5 (extra JSON field)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; rows shard across GPUs with no communication, "
+              "but no multi-GPU path is built or measured here. Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from approx_topk import _native
+
+    if not torch.cuda.is_available():
+        print("bench.py: needs a GPU", file=sys.stderr)
+        return 2
+    if not os.path.exists(_native.library_path()):
+        import __graft_entry__
+        __graft_entry__.build()
+
+    name = args.workload
+    rows, n, dtype, k, j, km, seed = CONFIGS[name]
+    xs, wall, dev_ms, elems, in_bytes = time_config(name, args.steps, args.warmup, args.inputs)
+    ms_per_step = wall * 1e3 / args.steps
+    launch_ms = dev_ms / args.steps  # device time between HIP events on the launch stream
+    rec, ok, checked = parity_and_recall(name, xs[0], 4)
+    esize = in_bytes // elems
+    out_bytes = rows * k * (esize + 8)
+
+    result = {
+        "metric": f"input HBM GB/s at {dtype} [{rows},{n}] k={k} j={j} k_mult={km}",
+        "value": in_bytes / (wall / args.steps) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if dtype == "float32" else "f16",
+        "data": "synthetic",
+        "config": {"workload": f"{name}: {dtype} x[{rows},{n}] iid N(0,1), k={k}, j={j}, k_mult={km}, "
+                               f"interleaved buckets, {len(xs)} rotating inputs resident in HBM"},
+        "elements_per_s": elems / (wall / args.steps),
+        "frac_of_hbm_peak": in_bytes / (wall / args.steps) / 1e9 / HBM_PEAK_GBS,
+        "input_plus_output_GBps": (in_bytes + out_bytes) / (wall / args.steps) / 1e9,
+        "recall_at_k": rec,
+        "oracle_bit_exact": ok,
+        "oracle_rows_checked": checked,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": in_bytes / (launch_ms * 1e-3) / 1e9,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": in_bytes / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "traffic": None,
+            "launch_us": launch_ms * 1e3,
+            "algorithmic_bytes_per_launch": in_bytes,
+        },
+    }
+    del xs
+    torch.cuda.empty_cache()
+
+    if args.all_configs:
+        others = {}
+        for other in ("C3", "C4", "C5"):
+            o_rows, o_n, o_dtype, o_k, o_j, o_km, _ = CONFIGS[other]
+            oxs, o_wall, o_dev_ms, o_elems, o_bytes = time_config(other, args.steps, args.warmup, args.inputs)
+            o_rec, o_ok, o_checked = parity_and_recall(other, oxs[0], 2)
+            others[other] = {
+                "shape": [o_rows, o_n], "dtype": o_dtype, "k": o_k, "j": o_j, "k_mult": o_km,
+                "us_per_step": o_dev_ms * 1e3 / args.steps,
+                "input_GBps": o_bytes / (o_dev_ms * 1e-3 / args.steps) / 1e9,
+                "frac_of_hbm_peak": o_bytes / (o_dev_ms * 1e-3 / args.steps) / 1e9 / HBM_PEAK_GBS,
+                "elements_per_s": o_elems / (o_dev_ms * 1e-3 / args.steps),
+                "recall_at_k": o_rec, "oracle_bit_exact": o_ok, "oracle_rows_checked": o_checked,
+            }
+            del oxs
+            torch.cuda.empty_cache()
+        result["other_configs"] = others
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(name)
+    print(json.dumps(result))
+    return 0 if ok else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())
