@@ -23,18 +23,37 @@ int check_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int
   return ATK_OK;
 }
 
+// Workspace of atk_topk: the stage-1 candidates, then stage 1's own scratch.
 struct TopkPlan {
-  size_t cand_values_off, cand_indices_off, total;
+  size_t cand_values_off, cand_indices_off, stage1_off, stage1_bytes, total;
 };
 
-TopkPlan plan_topk(int64_t rows, int64_t k0, int64_t k, int dtype) {
-  TopkPlan p{0, 0, 0};
-  if (k == k0 || rows <= 0 || k0 <= 0) return p;
+TopkPlan plan_topk(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype) {
+  TopkPlan p{0, 0, 0, 0, 0};
+  if (rows <= 0 || k0 <= 0) return p;
+  p.stage1_bytes = atk_stage1_workspace_bytes(rows, n, k0, j, layout, dtype);
+  if (k == k0) {
+    p.total = p.stage1_bytes;
+    return p;
+  }
   const size_t vals = align_up((size_t)rows * (size_t)k0 * atk::elem_bytes(dtype), 256);
-  p.cand_values_off = 0;
   p.cand_indices_off = vals;
-  p.total = vals + align_up((size_t)rows * (size_t)k0 * sizeof(int64_t), 256);
+  p.stage1_off = vals + align_up((size_t)rows * (size_t)k0 * sizeof(int64_t), 256);
+  p.total = p.stage1_off + p.stage1_bytes;
   return p;
+}
+
+// Stage 1 through the streaming kernels when they take the shape, else the
+// general kernel.
+int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+               int layout, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+               hipStream_t stream) {
+  bool handled = false;
+  const int rc = atk::launch_stage1_stream(x, rows, n, row_stride, k0, j, layout, dtype, values,
+                                           indices, ws, ws_bytes, stream, &handled);
+  if (handled || rc != ATK_OK) return rc;
+  return atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout, dtype, values,
+                                            indices, stream);
 }
 
 }  // namespace
@@ -58,16 +77,17 @@ const char* atk_strerror(int status) {
   return "unknown status";
 }
 
-size_t atk_stage1_workspace_bytes(int64_t, int64_t, int64_t, int, int, int) { return 0; }
+size_t atk_stage1_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype) {
+  return atk::stage1_stream_workspace_bytes(rows, n, k0, j, layout, dtype);
+}
 
 int atk_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
                int layout, int dtype, void* values, int64_t* indices, void* ws,
                size_t ws_bytes, atk_stream_t stream) {
-  (void)ws; (void)ws_bytes;
   const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices);
   if (rc != ATK_OK || k0 == 0 || rows == 0) return rc;
-  return atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout, dtype,
-                                            values, indices, (hipStream_t)stream);
+  return run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws, ws_bytes,
+                    (hipStream_t)stream);
 }
 
 size_t atk_select_workspace_bytes(int64_t, int64_t, int64_t, int) { return 0; }
@@ -86,8 +106,7 @@ int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t row
 
 size_t atk_topk_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int64_t k,
                                 int layout, int dtype) {
-  (void)n; (void)j; (void)layout;
-  return plan_topk(rows, k0, k, dtype).total;
+  return plan_topk(rows, n, k0, j, k, layout, dtype).total;
 }
 
 int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
@@ -99,14 +118,14 @@ int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t
   if (k == k0)
     return atk_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws,
                       ws_bytes, stream);
-  const TopkPlan p = plan_topk(rows, k0, k, dtype);
+  const TopkPlan p = plan_topk(rows, n, k0, j, k, layout, dtype);
   if (!ws || ws_bytes < p.total) return ATK_ERR_WORKSPACE;
   unsigned char* base = static_cast<unsigned char*>(ws);
   void* cand_values = base + p.cand_values_off;
   int64_t* cand_indices = reinterpret_cast<int64_t*>(base + p.cand_indices_off);
-  const int rc1 = atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout,
-                                                     dtype, cand_values, cand_indices,
-                                                     (hipStream_t)stream);
+  const int rc1 = run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, cand_values,
+                             cand_indices, base + p.stage1_off, p.stage1_bytes,
+                             (hipStream_t)stream);
   if (rc1 != ATK_OK) return rc1;
   const int64_t bound = (layout == ATK_CEIL_CHUNK || layout == ATK_INTERLEAVED_PADDED)
                             ? ((n + k0 - 1) / k0) * k0

@@ -14,6 +14,14 @@ int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
                                   int dtype, void* values, int64_t* indices,
                                   hipStream_t stream);
 
+// stage1_stream_plan.hip: interleaved layouts with at least j full sub-rows.
+// `*handled` tells whether the shape was accepted; if not, nothing was enqueued.
+size_t stage1_stream_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout,
+                                     int dtype);
+int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0,
+                         int j, int layout, int dtype, void* values, int64_t* indices, void* ws,
+                         size_t ws_bytes, hipStream_t stream, bool* handled);
+
 // stage2_radix_select.hip: one workgroup per row.
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,

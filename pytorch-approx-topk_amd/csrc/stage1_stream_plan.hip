@@ -1,0 +1,88 @@
+// Host-side planning and dispatch of the streaming stage-1 kernels.
+#include "stage1_stream.h"
+
+namespace atk {
+namespace stream {
+
+namespace {
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Waves wanted in flight: 256 CUs x 4 SIMDs x 4 waves.
+constexpr int64_t kTargetWaves = 4096;
+// Fewest sub-rows worth giving to one wave.
+constexpr int64_t kMinRun = 16;
+}  // namespace
+
+Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned) {
+  Plan pl{};
+  pl.ok = false;
+  if (layout != ATK_INTERLEAVED && layout != ATK_INTERLEAVED_PADDED) return pl;
+  if (rows <= 0 || k0 <= 0 || j < 1 || j > 4 || k0 % j) return pl;
+  const int es = elem_bytes(dtype);
+  if (!es) return pl;
+  const int64_t b = k0 / j;
+  const int64_t full = n / b;
+  if (full < j || full > 0xffffffffll || b > 0x7fffffffll) return pl;
+  pl.full_rows = (uint32_t)full;
+  pl.rem = (uint32_t)(n - full * b);
+  pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
+  const int vf = 16 / es;
+  pl.vec = (aligned && b % vf == 0) ? vf : 1;
+
+  const int64_t tile_cols = (int64_t)kWave * pl.vec;
+  const int64_t wave_tiles = (b + tile_cols - 1) / tile_cols;
+  const int64_t waves = rows * wave_tiles;
+  pl.split_wg = false;
+  pl.slabs = 1;
+  if (waves < kTargetWaves / 2 && full >= (int64_t)kWavesPerGroup * j * 2) {
+    pl.split_wg = true;
+    const int64_t min_run = j > kMinRun ? j : kMinRun;
+    const int64_t want = (kTargetWaves + waves - 1) / waves;         // total split factor wanted
+    int64_t slabs = (want + kWavesPerGroup - 1) / kWavesPerGroup;
+    const int64_t most = full / (kWavesPerGroup * min_run);          // slabs the row can feed
+    if (slabs > most) slabs = most;
+    if (slabs < 1) slabs = 1;
+    pl.slabs = (uint32_t)slabs;
+  }
+  pl.slab_len = (uint32_t)(full / pl.slabs);
+  pl.col_tiles = (uint32_t)(pl.split_wg ? wave_tiles : (wave_tiles + kWavesPerGroup - 1) / kWavesPerGroup);
+  if (pl.slabs > 1) {
+    const size_t entries = (size_t)rows * pl.slabs * (size_t)k0;
+    pl.part_values_off = 0;
+    pl.part_pos_off = align_up(entries * es, 256);
+    pl.ws_bytes = pl.part_pos_off + align_up(entries * sizeof(uint32_t), 256);
+  }
+  pl.ok = true;
+  return pl;
+}
+
+}  // namespace stream
+
+size_t stage1_stream_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype) {
+  const stream::Plan a = stream::make_plan(rows, n, k0, j, layout, dtype, true);
+  const stream::Plan u = stream::make_plan(rows, n, k0, j, layout, dtype, false);
+  size_t need = 0;
+  if (a.ok && a.ws_bytes > need) need = a.ws_bytes;
+  if (u.ok && u.ws_bytes > need) need = u.ws_bytes;
+  return need;
+}
+
+int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                         int layout, int dtype, void* values, int64_t* indices, void* ws,
+                         size_t ws_bytes, hipStream_t stream, bool* handled) {
+  const int es = elem_bytes(dtype);
+  const int vf = es ? 16 / es : 1;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)values % 16 == 0) &&
+                       ((uintptr_t)indices % 16 == 0) && (row_stride % vf == 0);
+  const stream::Plan pl = stream::make_plan(rows, n, k0, j, layout, dtype, aligned);
+  *handled = pl.ok;
+  if (!pl.ok) return ATK_OK;
+  if (pl.ws_bytes && (!ws || ws_bytes < pl.ws_bytes || (uintptr_t)ws % 16 != 0)) return ATK_ERR_WORKSPACE;
+  int rc = ATK_ERR_DTYPE;
+  ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
+                   rc = stream::launch_typed<E>(pl, x, rows, row_stride, k0 / j, j, values, indices, ws,
+                                                stream));
+  return rc;
+}
+
+}  // namespace atk
