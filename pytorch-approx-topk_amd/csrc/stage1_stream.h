@@ -11,12 +11,13 @@
 // registers: values in compare form plus the sub-row number they came from; the
 // position in the row, c + p*b, is formed only when results are written.
 //
-// Work split.  Sub-rows are cut into `slabs` (grid dimension) so that short,
-// wide batches and long single rows both fill the machine.  Inside a workgroup
-// of 4 waves either every wave takes its own column tile (SPLIT_WG = false) or
-// the four waves share one column tile and each scans a quarter of the slab,
-// merging through LDS (SPLIT_WG = true).  With more than one slab the per-slab
-// queues go to a workspace and `stream_merge_kernel` folds them.
+// Work split.  A workgroup of W waves owns one column tile (64*V columns) over
+// one slab of sub-rows; each wave scans 1/W of the slab and waves 1..W-1 hand
+// their queues to wave 0 through LDS.  Many short-lived waves keep far more of
+// the HBM bandwidth than few long-lived ones on this part, and the merge is a
+// handful of register operations.  Very long rows are additionally cut into
+// `slabs` along the grid; then the per-slab queues go to a workspace and
+// `stream_merge_kernel` folds them.
 //
 // Order.  Sub-rows are visited in increasing position and a newcomer displaces
 // an entry only when it compares strictly greater, so equal values keep the
@@ -27,6 +28,7 @@
 #pragma once
 
 #include <type_traits>
+#include <utility>
 
 #include "atk_device.h"
 #include "atk_launch.h"
@@ -35,8 +37,17 @@ namespace atk {
 namespace stream {
 
 constexpr int kWave = 64;
-constexpr int kWavesPerGroup = 4;
-constexpr int kGroup = kWave * kWavesPerGroup;
+
+// Columns per lane with vector loads: 16 bytes' worth, but at most 8 columns so
+// that the queues of one lane stay in registers.
+__host__ __device__ constexpr int full_vec(int elem_size) { return elem_size == 1 ? 8 : 16 / elem_size; }
+
+// LDS a workgroup of `waves` needs to hand the queues of waves 1.. to wave 0,
+// and the most the planner lets it use.
+__host__ __device__ constexpr size_t merge_lds_bytes(int vec, int j, int waves, int cmp_size) {
+  return (size_t)(waves - 1) * vec * j * kWave * (cmp_size + 4);
+}
+constexpr size_t kMergeLdsLimit = 48 * 1024;
 
 // ---------------------------------------------------------------------------
 // Compare form of an element type: what the queues hold in the hot loop.
@@ -93,6 +104,15 @@ template <> struct Cmp<Elem<ATK_I64>> {
   __device__ static inline uint64_t to_raw(cmp_t v) { return (uint64_t)v; }
 };
 
+// Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).
+template <typename F, int... I>
+__device__ inline void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ inline void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 // V elements moved by one load instruction.
 template <typename raw_t, int V> struct alignas(sizeof(raw_t) * V) Pack { raw_t e[V]; };
 
@@ -135,8 +155,8 @@ __device__ inline void push_exact(typename E::raw_t (&q)[J], uint32_t (&pos)[J],
   if (filled < J) ++filled;
 }
 
-struct Args {
-  const void* x;          // input rows
+// Shape of one launch; passed to the kernels by value.
+struct Geom {
   int64_t row_stride;     // elements between rows
   int64_t b;              // buckets (columns) per row
   uint32_t full_rows;     // L = n / b
@@ -145,22 +165,28 @@ struct Args {
   uint32_t slabs;         // sub-row slabs per row
   uint32_t slab_len;      // sub-rows per slab (the last slab takes the rest)
   uint32_t col_tiles;     // workgroup column tiles per row
-  void* values;           // slabs == 1: final values[rows][b*J]
-  int64_t* indices;       //             final indices
-  void* part_values;      // slabs > 1: [rows][slabs][b*J] raw values
-  uint32_t* part_pos;     //            and their sub-row numbers
+};
+
+// Where results go: final values/indices[rows][b*J] when there is one slab,
+// else per-slab queues [rows][slabs][b*J] (raw values and sub-row numbers).
+template <typename raw_t> struct Sink {
+  raw_t* values;
+  int64_t* indices;
+  raw_t* part_values;
+  uint32_t* part_pos;
 };
 
 // Writes the queues of this lane's V columns, either as final results or as a
 // slab's partial result.
 template <typename E, int J, int V>
-__device__ inline void emit(const Args& a, int64_t row, uint32_t slab, int64_t col,
-                            const typename E::raw_t (&val)[V][J], const uint32_t (&pos)[V][J]) {
+__device__ inline void emit(const Geom& g, const Sink<typename E::raw_t>& out, int64_t row,
+                            uint32_t slab, int64_t col, const typename E::raw_t (&val)[V][J],
+                            const uint32_t (&pos)[V][J]) {
   using raw_t = typename E::raw_t;
-  if (a.slabs == 1) {
-    const int64_t o = (row * a.b + col) * J;
-    raw_t* ov = static_cast<raw_t*>(a.values) + o;
-    int64_t* oi = a.indices + o;
+  if (g.slabs == 1) {
+    const int64_t o = (row * g.b + col) * J;
+    raw_t* ov = out.values + o;
+    int64_t* oi = out.indices + o;
     if constexpr (V > 1) {
       // V*J values = J 16-byte stores; V*J int64 = V*J/2 16-byte stores
       Pack<raw_t, V> pv[J];
@@ -170,7 +196,7 @@ __device__ inline void emit(const Args& a, int64_t row, uint32_t slab, int64_t c
 #pragma unroll
         for (int s = 0; s < J; ++s) {
           pv[(v * J + s) / V].e[(v * J + s) % V] = val[v][s];
-          pi[(v * J + s) / 2].e[(v * J + s) % 2] = col + v + (int64_t)pos[v][s] * a.b;
+          pi[(v * J + s) / 2].e[(v * J + s) % 2] = col + v + (int64_t)pos[v][s] * g.b;
         }
 #pragma unroll
       for (int t = 0; t < J; ++t) reinterpret_cast<Pack<raw_t, V>*>(ov)[t] = pv[t];
@@ -178,12 +204,12 @@ __device__ inline void emit(const Args& a, int64_t row, uint32_t slab, int64_t c
       for (int t = 0; t < V * J / 2; ++t) reinterpret_cast<Pack<int64_t, 2>*>(oi)[t] = pi[t];
     } else {
 #pragma unroll
-      for (int s = 0; s < J; ++s) { ov[s] = val[0][s]; oi[s] = col + (int64_t)pos[0][s] * a.b; }
+      for (int s = 0; s < J; ++s) { ov[s] = val[0][s]; oi[s] = col + (int64_t)pos[0][s] * g.b; }
     }
   } else {
-    const int64_t o = ((row * a.slabs + slab) * a.b + col) * J;
-    raw_t* ov = static_cast<raw_t*>(a.part_values) + o;
-    uint32_t* op = a.part_pos + o;
+    const int64_t o = ((row * g.slabs + slab) * g.b + col) * J;
+    raw_t* ov = out.part_values + o;
+    uint32_t* op = out.part_pos + o;
 #pragma unroll
     for (int v = 0; v < V; ++v)
 #pragma unroll
@@ -194,63 +220,84 @@ __device__ inline void emit(const Args& a, int64_t row, uint32_t slab, int64_t c
 // Exact recomputation of one lane's V columns over sub-rows [p0, p1) (plus the
 // partial sub-row when `with_rem`), through order keys.  Off the hot path.
 template <typename E, int J, int V>
-__device__ __noinline__ void exact_columns(const Args& a, int64_t row, uint32_t slab, int64_t col,
-                                           uint32_t p0, uint32_t p1, bool with_rem) {
+__device__ inline void exact_columns(const typename E::raw_t* __restrict__ xr, const Geom& g,
+                                     const Sink<typename E::raw_t>& out, int64_t row, uint32_t slab,
+                                     int64_t col, uint32_t p0, uint32_t p1, bool with_rem) {
   using raw_t = typename E::raw_t;
-  const raw_t* xr = static_cast<const raw_t*>(a.x) + row * a.row_stride;
   raw_t val[V][J];
   uint32_t pos[V][J];
 #pragma unroll
-  for (int v = 0; v < V; ++v) {
-    int filled = 0;
+  for (int v = 0; v < V; ++v)
 #pragma unroll
     for (int s = 0; s < J; ++s) { val[v][s] = 0; pos[v][s] = 0; }
-    for (uint32_t p = p0; p < p1; ++p)
-      push_exact<E, J>(val[v], pos[v], filled, xr[(int64_t)p * a.b + col + v], p);
-    if (with_rem && a.rem != 0) {
-      if (col + v < (int64_t)a.rem)
-        push_exact<E, J>(val[v], pos[v], filled, xr[(int64_t)a.full_rows * a.b + col + v], a.full_rows);
-      else if (a.pad_tail)
-        push_exact<E, J>(val[v], pos[v], filled, E::pad_raw, a.full_rows);
+  int filled = 0;  // the V columns fill in step
+  for (uint32_t p = p0; p < p1; ++p) {
+    int f = filled;
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      f = filled;
+      push_exact<E, J>(val[v], pos[v], f, xr[(int64_t)p * g.b + col + v], p);
+    }
+    filled = f;
+  }
+  if (with_rem && g.rem != 0) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      int f = filled;
+      if (col + v < (int64_t)g.rem)
+        push_exact<E, J>(val[v], pos[v], f, xr[(int64_t)g.full_rows * g.b + col + v], g.full_rows);
+      else if (g.pad_tail)
+        push_exact<E, J>(val[v], pos[v], f, E::pad_raw, g.full_rows);
     }
   }
-  emit<E, J, V>(a, row, slab, col, val, pos);
+  emit<E, J, V>(g, out, row, slab, col, val, pos);
 }
 
-template <typename E, int J, int V, bool SPLIT_WG, int U>
-__global__ __launch_bounds__(kGroup) void stream_kernel(const Args a) {
+// E: element traits; J: entries kept per bucket; V: columns per lane; W: waves
+// per workgroup, sharing one column tile and splitting its sub-rows; U: loads
+// kept in flight per lane.
+template <typename E, int J, int V, int W, int U>
+__global__ __launch_bounds__(kWave * W) void stream_kernel(
+    const typename E::raw_t* __restrict__ x, const Sink<typename E::raw_t> out, const Geom g) {
   using raw_t = typename E::raw_t;
   using C = Cmp<E>;
   using cmp_t = typename C::cmp_t;
-  constexpr int kTileCols = kWave * V;                                  // columns per wave
-  constexpr int kGroupCols = SPLIT_WG ? kTileCols : kTileCols * kWavesPerGroup;
+  static_assert(U >= J, "the first U loads must cover the J sub-rows that fill the queues");
+  constexpr int kTileCols = kWave * V;
 
-  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const uint32_t lane = threadIdx.x % kWave;
+  // Everything that decides control flow is wave-uniform; say so, so that it
+  // lives in scalar registers.
+  const uint32_t wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) : 0;
   uint32_t blk = blockIdx.x;
-  const uint32_t col_tile = blk % a.col_tiles; blk /= a.col_tiles;
-  const uint32_t slab = blk % a.slabs;
-  const int64_t row = blk / a.slabs;
+  const uint32_t col_tile = __builtin_amdgcn_readfirstlane(blk % g.col_tiles);
+  blk /= g.col_tiles;
+  const uint32_t slab = __builtin_amdgcn_readfirstlane(blk % g.slabs);
+  const int64_t row = __builtin_amdgcn_readfirstlane(blk / g.slabs);
 
-  const int64_t col = (int64_t)col_tile * kGroupCols + (SPLIT_WG ? 0 : wave * kTileCols) + lane * V;
-  const bool live = col < a.b;  // b is a multiple of V whenever V > 1
+  const int64_t col = (int64_t)col_tile * kTileCols + lane * V;
+  const bool live = col < g.b;  // b is a multiple of V whenever V > 1
 
-  // sub-rows of this slab, then of this wave
-  uint32_t p0 = slab * a.slab_len;
-  uint32_t p1 = (slab + 1 == a.slabs) ? a.full_rows : p0 + a.slab_len;
-  const uint32_t s0 = p0, s1 = p1;
-  if (SPLIT_WG) {
-    const uint32_t len = p1 - p0;
-    p1 = p0 + (uint32_t)(((uint64_t)len * (wave + 1)) / kWavesPerGroup);
-    p0 = p0 + (uint32_t)(((uint64_t)len * wave) / kWavesPerGroup);
-  }
-  const bool last_run = (slab + 1 == a.slabs) && (!SPLIT_WG || wave == kWavesPerGroup - 1);
+  // sub-rows of this slab [s0, s1), then of this wave [p0, p1)
+  const uint32_t s0 = slab * g.slab_len;
+  const uint32_t s1 = (slab + 1 == g.slabs) ? g.full_rows : s0 + g.slab_len;
+  const uint32_t p0 = __builtin_amdgcn_readfirstlane(s0 + (uint32_t)(((uint64_t)(s1 - s0) * wave) / W));
+  const uint32_t p1 = __builtin_amdgcn_readfirstlane(s0 + (uint32_t)(((uint64_t)(s1 - s0) * (wave + 1)) / W));
+  const bool last_slab = slab + 1 == g.slabs;
+  const bool last_run = last_slab && wave == W - 1;
 
-  const raw_t* xr = static_cast<const raw_t*>(a.x) + row * a.row_stride;
-  const raw_t* src = xr + (live ? col : 0);
+  const raw_t* xr = x + row * g.row_stride;
+  // `next` walks down this lane's columns one sub-row per load
+  const raw_t* next = xr + (live ? col : 0) + (int64_t)p0 * g.b;
+  auto load_next = [&]() {
+    const Pack<raw_t, V> pk = load_pack<raw_t, V>(next);
+    next += g.b;
+    return pk;
+  };
 
   cmp_t q[V][J];
   uint32_t pos[V][J];
-  bool nan_seen = false;
+  uint64_t nan_mask = 0;  // lanes that saw a NaN; wave-uniform
 
   auto take = [&](const Pack<raw_t, V>& pk, uint32_t p, auto filled_tag) {
     constexpr int FILLED = decltype(filled_tag)::value;
@@ -259,62 +306,73 @@ __global__ __launch_bounds__(kGroup) void stream_kernel(const Args a) {
     for (int v = 0; v < V; ++v) c[v] = C::from_raw(pk.e[v]);
     if constexpr (C::has_nan) {
 #pragma unroll
-      for (int v = 0; v + 1 < V; v += 2) nan_seen |= __builtin_isunordered(c[v], c[v + 1]);
-      if constexpr (V % 2 != 0) nan_seen |= __builtin_isunordered(c[V - 1], c[V - 1]);
+      for (int v = 0; v + 1 < V; v += 2) nan_mask |= __ballot(__builtin_isunordered(c[v], c[v + 1]));
+      if constexpr (V % 2 != 0) nan_mask |= __ballot(__builtin_isunordered(c[V - 1], c[V - 1]));
     }
 #pragma unroll
     for (int v = 0; v < V; ++v) push<cmp_t, J, FILLED>(q[v], pos[v], c[v], p);
   };
 
-  // first J sub-rows fill the queues
-  {
-    Pack<raw_t, V> first[J];
+  // U loads stay in flight.  Slot u of `buf` holds sub-row p + u; consuming it
+  // frees the slot for sub-row p + U + u.  `ld` is the next sub-row to load.
+  Pack<raw_t, V> buf[U];
+  uint32_t ld = p0;
 #pragma unroll
-    for (int t = 0; t < J; ++t) first[t] = load_pack<raw_t, V>(src + (int64_t)(p0 + t) * a.b);
-    take(first[0], p0, std::integral_constant<int, 0>{});
-    if constexpr (J > 1) take(first[1], p0 + 1, std::integral_constant<int, 1>{});
-    if constexpr (J > 2) take(first[2], p0 + 2, std::integral_constant<int, 2>{});
-    if constexpr (J > 3) take(first[3], p0 + 3, std::integral_constant<int, 3>{});
+  for (int u = 0; u < U; ++u) {
+    if (ld < p1) { buf[u] = load_next(); ++ld; }
   }
-  uint32_t p = p0 + J;
-  const raw_t* cur = src + (int64_t)p * a.b;
-  for (; p + U <= p1; p += U) {
-    Pack<raw_t, V> buf[U];
+  uint32_t p = p0;
+  // first group: also fills the queues (the run has at least J sub-rows)
+  static_for<U>([&](auto uc) {
+    constexpr int u = decltype(uc)::value;
+    if (p0 + u < p1) {
+      const Pack<raw_t, V> cur = buf[u];
+      if (ld < p1) { buf[u] = load_next(); ++ld; }
+      take(cur, p0 + u, std::integral_constant<int, (u < J ? u : J)>{});
+    }
+  });
+  p += U;
+  // steady state: every slot is consumed and refilled
+  while (ld + U <= p1) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) buf[u] = load_pack<raw_t, V>(cur + (int64_t)u * a.b);
-    cur += (int64_t)U * a.b;
-#pragma unroll
-    for (int u = 0; u < U; ++u) take(buf[u], p + u, std::integral_constant<int, J>{});
+    for (int u = 0; u < U; ++u) {
+      const Pack<raw_t, V> cur = buf[u];
+      buf[u] = load_next();
+      take(cur, p + u, std::integral_constant<int, J>{});
+    }
+    p += U;
+    ld += U;
   }
-  for (; p < p1; ++p) {
-    const Pack<raw_t, V> one = load_pack<raw_t, V>(cur);
-    cur += a.b;
-    take(one, p, std::integral_constant<int, J>{});
+  // drain: at most two partly valid groups
+  for (; p < p1; p += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (p + u < p1) {
+        const Pack<raw_t, V> cur = buf[u];
+        if (ld < p1) { buf[u] = load_next(); ++ld; }
+        take(cur, p + u, std::integral_constant<int, J>{});
+      }
+    }
   }
   // the partial sub-row: column c has one more element when c < rem
   // (with a padded row the other columns see the pad value there)
-  if (last_run && a.rem != 0) {
+  if (last_run && g.rem != 0) {
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-      const bool real = col + v < (int64_t)a.rem;
-      if (live && (real || a.pad_tail)) {
-        const cmp_t c = C::from_raw(real ? xr[(int64_t)a.full_rows * a.b + col + v] : E::pad_raw);
-        if constexpr (C::has_nan) nan_seen |= __builtin_isunordered(c, c);
-        push<cmp_t, J, J>(q[v], pos[v], c, a.full_rows);
+      const bool real = col + v < (int64_t)g.rem;
+      if (live && (real || g.pad_tail)) {
+        const cmp_t c = C::from_raw(real ? xr[(int64_t)g.full_rows * g.b + col + v] : E::pad_raw);
+        if constexpr (C::has_nan) nan_mask |= __ballot(__builtin_isunordered(c, c));
+        push<cmp_t, J, J>(q[v], pos[v], c, g.full_rows);
       }
     }
   }
 
-  raw_t val[V][J];
-  if constexpr (!SPLIT_WG) {
-    if (C::has_nan && __any(nan_seen)) {
-      if (live) exact_columns<E, J, V>(a, row, slab, col, p0, p1, last_run);
-      return;
-    }
-  } else {
-    // waves 1..3 hand their queues to wave 0 through LDS, in sub-row order
-    __shared__ cmp_t lds_q[kWavesPerGroup - 1][V * J][kWave];
-    __shared__ uint32_t lds_p[kWavesPerGroup - 1][V * J][kWave];
+  bool any_nan = C::has_nan && nan_mask != 0;
+  if constexpr (W > 1) {
+    // waves 1.. hand their queues to wave 0 through LDS
+    __shared__ cmp_t lds_q[W - 1][V * J][kWave];
+    __shared__ uint32_t lds_p[W - 1][V * J][kWave];
     if (wave > 0) {
 #pragma unroll
       for (int v = 0; v < V; ++v)
@@ -324,26 +382,35 @@ __global__ __launch_bounds__(kGroup) void stream_kernel(const Args a) {
           lds_p[wave - 1][v * J + s][lane] = pos[v][s];
         }
     }
-    const int any_nan = __syncthreads_or(C::has_nan && nan_seen);
-    if (wave > 0) return;
-    if (any_nan) {
-      if (live) exact_columns<E, J, V>(a, row, slab, col, s0, s1, slab + 1 == a.slabs);
-      return;
+    if constexpr (C::has_nan) {
+      any_nan = __syncthreads_or(any_nan);
+    } else {
+      __syncthreads();
     }
+    if (wave > 0) return;
+    if (!any_nan) {
+      // fold in sub-row order, each wave's entries best first, so that equal
+      // values keep the lowest index
+#pragma nounroll
+      for (int w = 0; w < W - 1; ++w)
 #pragma unroll
-    for (int w = 0; w < kWavesPerGroup - 1; ++w)
+        for (int v = 0; v < V; ++v)
 #pragma unroll
-      for (int v = 0; v < V; ++v)
-#pragma unroll
-        for (int s = J - 1; s >= 0; --s)  // best entry first keeps equal values in index order
-          push<cmp_t, J, J>(q[v], pos[v], lds_q[w][v * J + s][lane], lds_p[w][v * J + s][lane]);
+          for (int s = J - 1; s >= 0; --s)
+            push<cmp_t, J, J>(q[v], pos[v], lds_q[w][v * J + s][lane], lds_p[w][v * J + s][lane]);
+    }
   }
   if (!live) return;
+  if (any_nan) {
+    exact_columns<E, J, V>(xr, g, out, row, slab, col, s0, W > 1 ? s1 : p1, last_slab);
+    return;
+  }
+  raw_t val[V][J];
 #pragma unroll
   for (int v = 0; v < V; ++v)
 #pragma unroll
     for (int s = 0; s < J; ++s) val[v][s] = C::to_raw(q[v][s]);
-  emit<E, J, V>(a, row, slab, col, val, pos);
+  emit<E, J, V>(g, out, row, slab, col, val, pos);
 }
 
 // Folds the per-slab queues of every bucket into the final result, one lane per
@@ -380,7 +447,7 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(
 struct Plan {
   bool ok;            // the streaming kernels accept this shape
   int vec;            // V: elements per load (16 bytes' worth, or 1)
-  bool split_wg;
+  int waves;          // W: waves per workgroup (1, 2, 4 or 8)
   uint32_t full_rows, rem, pad_tail;
   uint32_t slabs, slab_len, col_tiles;
   size_t part_values_off, part_pos_off, ws_bytes;

@@ -1,4 +1,6 @@
 // Host-side planning and dispatch of the streaming stage-1 kernels.
+#include <cstdlib>
+
 #include "stage1_stream.h"
 
 namespace atk {
@@ -7,10 +9,10 @@ namespace stream {
 namespace {
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Waves wanted in flight: 256 CUs x 4 SIMDs x 4 waves.
+// Waves wanted in the grid: a few per SIMD of the 256 CUs x 4 SIMDs.
 constexpr int64_t kTargetWaves = 4096;
-// Fewest sub-rows worth giving to one wave.
-constexpr int64_t kMinRun = 16;
+// Sub-rows worth giving to one wave before a row is also cut into slabs.
+constexpr int64_t kSlabRun = 16;
 }  // namespace
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned) {
@@ -26,26 +28,38 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   pl.full_rows = (uint32_t)full;
   pl.rem = (uint32_t)(n - full * b);
   pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
-  const int vf = 16 / es;
+  const int vf = full_vec(es);
   pl.vec = (aligned && b % vf == 0) ? vf : 1;
 
   const int64_t tile_cols = (int64_t)kWave * pl.vec;
-  const int64_t wave_tiles = (b + tile_cols - 1) / tile_cols;
-  const int64_t waves = rows * wave_tiles;
-  pl.split_wg = false;
+  pl.col_tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
+
+  // Waves per workgroup: as many as leave every wave at least max(j, 4)
+  // sub-rows and fit the LDS hand-over (entries are at most 8 + 4 bytes).
+  const int64_t min_run = j > 4 ? j : 4;
+  const int cmp_size = es > 4 ? 8 : 4;
+  int w = 8;
+  while (w > 1 && (full / w < min_run || merge_lds_bytes(pl.vec, j, w, cmp_size) > kMergeLdsLimit)) w /= 2;
+  pl.waves = w;
+
+  // Slabs: only when the grid would still be small and the runs are long.
   pl.slabs = 1;
-  if (waves < kTargetWaves / 2 && full >= (int64_t)kWavesPerGroup * j * 2) {
-    pl.split_wg = true;
-    const int64_t min_run = j > kMinRun ? j : kMinRun;
-    const int64_t want = (kTargetWaves + waves - 1) / waves;         // total split factor wanted
-    int64_t slabs = (want + kWavesPerGroup - 1) / kWavesPerGroup;
-    const int64_t most = full / (kWavesPerGroup * min_run);          // slabs the row can feed
+  const int64_t waves = rows * pl.col_tiles * w;
+  if (waves < kTargetWaves) {
+    int64_t slabs = (kTargetWaves + waves - 1) / waves;
+    const int64_t most = full / (w * kSlabRun);
     if (slabs > most) slabs = most;
     if (slabs < 1) slabs = 1;
     pl.slabs = (uint32_t)slabs;
   }
+  if (const char* e = getenv("ATK_TUNE_WAVES")) {
+    const int tw = atoi(e);
+    if ((tw == 1 || tw == 2 || tw == 4 || tw == 8) && full / tw >= j &&
+        merge_lds_bytes(pl.vec, j, tw, cmp_size) <= kMergeLdsLimit)
+      pl.waves = tw;
+    if (const char* s = getenv("ATK_TUNE_SLABS")) pl.slabs = (uint32_t)atoi(s);
+  }
   pl.slab_len = (uint32_t)(full / pl.slabs);
-  pl.col_tiles = (uint32_t)(pl.split_wg ? wave_tiles : (wave_tiles + kWavesPerGroup - 1) / kWavesPerGroup);
   if (pl.slabs > 1) {
     const size_t entries = (size_t)rows * pl.slabs * (size_t)k0;
     pl.part_values_off = 0;
@@ -71,7 +85,7 @@ int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_str
                          int layout, int dtype, void* values, int64_t* indices, void* ws,
                          size_t ws_bytes, hipStream_t stream, bool* handled) {
   const int es = elem_bytes(dtype);
-  const int vf = es ? 16 / es : 1;
+  const int vf = es ? stream::full_vec(es) : 1;
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)values % 16 == 0) &&
                        ((uintptr_t)indices % 16 == 0) && (row_stride % vf == 0);
   const stream::Plan pl = stream::make_plan(rows, n, k0, j, layout, dtype, aligned);
