@@ -25,6 +25,10 @@ for p in (ROOT, os.path.join(ROOT, "pytorch-approx-topk_amd")):
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of the headline kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
+# copy of known size (profiles/stream_kernel_f32_j2_c2_hbm_traffic.md); None for other workloads.
+MEASURED_TRAFFIC_BYTES = {"C2": 637_638_750}
+
 # name -> (rows, n, dtype, k, j, k_mult, seed)
 CONFIGS = {
     "C1": (4, 65536, "float32", 1024, 1, 1, 1001),
@@ -140,12 +144,16 @@ def cpu_baseline(name: str):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=150,
+                    help="untimed steps; the clocks of an idle GPU take ~100 launches to settle")
     ap.add_argument("--inputs", type=int, default=5, help="distinct input tensors to rotate over")
     ap.add_argument("--workload", default="C2", choices=sorted(CONFIGS))
     ap.add_argument("--all-configs", action="store_true", help="also time C3, C4, C5 (extra JSON field)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 512 MiB device copy a few times (a kernel of known traffic for "
+                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; rows shard across GPUs with no communication, "
@@ -199,13 +207,22 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": in_bytes / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(name),
             "launch_us": launch_ms * 1e3,
             "algorithmic_bytes_per_launch": in_bytes,
         },
     }
     del xs
     torch.cuda.empty_cache()
+
+    if args.calibrate_copy:
+        src = torch.randn(128 << 20, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     if args.all_configs:
         others = {}
