@@ -413,27 +413,52 @@ __global__ __launch_bounds__(kWave * W) void stream_kernel(
   emit<E, J, V>(g, out, row, slab, col, val, pos);
 }
 
-// Folds the per-slab queues of every bucket into the final result, one lane per
-// bucket, with exact order keys.  Slabs are visited in sub-row order and each
-// slab's entries best first, so equal values keep the lowest index.
+// Folds the per-slab queues of every bucket into the final result with exact
+// order keys.  A workgroup of 4 waves covers 64 buckets (one per lane); wave w
+// folds a contiguous quarter of the slabs, then waves 1..3 hand their queues to
+// wave 0 through LDS.  Slabs are visited in sub-row order and each queue's
+// entries best first, so equal values keep the lowest index.
+constexpr int kMergeWaves = 4;
+
 template <typename E, int J>
-__global__ __launch_bounds__(256) void stream_merge_kernel(
+__global__ __launch_bounds__(kWave * kMergeWaves) void stream_merge_kernel(
     const typename E::raw_t* __restrict__ part_values, const uint32_t* __restrict__ part_pos,
     int64_t b, uint32_t slabs, int64_t blocks_per_row, typename E::raw_t* __restrict__ values,
     int64_t* __restrict__ indices) {
   using raw_t = typename E::raw_t;
+  __shared__ raw_t lds_q[kMergeWaves - 1][J][kWave];
+  __shared__ uint32_t lds_p[kMergeWaves - 1][J][kWave];
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int64_t row = blockIdx.x / blocks_per_row;
-  const int64_t c = (blockIdx.x - row * blocks_per_row) * 256 + threadIdx.x;
-  if (c >= b) return;
+  const int64_t c = (blockIdx.x - row * blocks_per_row) * kWave + lane;
+  const bool live = c < b;
   raw_t q[J];
   uint32_t pos[J];
   int filled = 0;
 #pragma unroll
   for (int s = 0; s < J; ++s) { q[s] = 0; pos[s] = 0; }
-  for (uint32_t slab = 0; slab < slabs; ++slab) {
-    const int64_t o = ((row * slabs + slab) * b + c) * J;
+  const uint32_t lo = (uint32_t)(((uint64_t)slabs * wave) / kMergeWaves);
+  const uint32_t hi = (uint32_t)(((uint64_t)slabs * (wave + 1)) / kMergeWaves);
+  if (live) {
+    for (uint32_t slab = lo; slab < hi; ++slab) {
+      const int64_t o = ((row * slabs + slab) * b + c) * J;
 #pragma unroll
-    for (int s = J - 1; s >= 0; --s) push_exact<E, J>(q, pos, filled, part_values[o + s], part_pos[o + s]);
+      for (int s = J - 1; s >= 0; --s) push_exact<E, J>(q, pos, filled, part_values[o + s], part_pos[o + s]);
+    }
+  }
+  // a wave whose quarter is empty hands over nothing; all lanes of a wave agree on `filled`
+  if (wave > 0) {
+#pragma unroll
+    for (int s = 0; s < J; ++s) { lds_q[wave - 1][s][lane] = q[s]; lds_p[wave - 1][s][lane] = pos[s]; }
+  }
+  __syncthreads();
+  if (wave > 0 || !live) return;
+  for (int w = 1; w < kMergeWaves; ++w) {
+    const uint32_t wlo = (uint32_t)(((uint64_t)slabs * w) / kMergeWaves);
+    const uint32_t whi = (uint32_t)(((uint64_t)slabs * (w + 1)) / kMergeWaves);
+    if (whi == wlo) continue;  // that wave had no slab
+#pragma unroll
+    for (int s = J - 1; s >= 0; --s) push_exact<E, J>(q, pos, filled, lds_q[w - 1][s][lane], lds_p[w - 1][s][lane]);
   }
   const int64_t o = (row * b + c) * J;
 #pragma unroll

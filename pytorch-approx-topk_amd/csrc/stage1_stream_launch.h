@@ -43,9 +43,10 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
   const int rc = pl.vec > 1 ? launch_w<E, J, VF>(pl, x, out, g, rows, stream)
                             : launch_w<E, J, 1>(pl, x, out, g, rows, stream);
   if (rc != ATK_OK || pl.slabs == 1) return rc;
-  const int64_t blocks_per_row = (g.b + 255) / 256;
+  const int64_t blocks_per_row = (g.b + kWave - 1) / kWave;
   if (blocks_per_row * rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
-  hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)), dim3(256), 0,
+  hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)),
+                     dim3(kWave * kMergeWaves), 0,
                      stream, (const raw_t*)out.part_values, (const uint32_t*)out.part_pos, g.b, pl.slabs,
                      blocks_per_row, out.values, out.indices);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;

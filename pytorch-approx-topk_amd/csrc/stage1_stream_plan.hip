@@ -9,8 +9,9 @@ namespace stream {
 namespace {
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Waves wanted in the grid: a few per SIMD of the 256 CUs x 4 SIMDs.
-constexpr int64_t kTargetWaves = 4096;
+// Waves wanted in the grid before a row is cut into slabs: one per SIMD of the
+// 256 CUs x 4 SIMDs (each keeps 8 KiB of loads in flight).
+constexpr int64_t kTargetWaves = 1024;
 // Sub-rows worth giving to one wave before a row is also cut into slabs.
 constexpr int64_t kSlabRun = 16;
 }  // namespace
@@ -34,12 +35,19 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   const int64_t tile_cols = (int64_t)kWave * pl.vec;
   pl.col_tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
 
-  // Waves per workgroup: as many as leave every wave at least max(j, 4)
-  // sub-rows and fit the LDS hand-over (entries are at most 8 + 4 bytes).
-  const int64_t min_run = j > 4 ? j : 4;
+  // Waves per workgroup.  Wave 0's serial work per column is its own run,
+  // full/w pushes, plus (w-1)*j pushes to fold the other waves' queues; take
+  // the w that minimises it (the larger on a tie: short-lived waves keep more
+  // of the HBM bandwidth), with every run at least j long and the LDS
+  // hand-over within its budget.
   const int cmp_size = es > 4 ? 8 : 4;
-  int w = 8;
-  while (w > 1 && (full / w < min_run || merge_lds_bytes(pl.vec, j, w, cmp_size) > kMergeLdsLimit)) w /= 2;
+  int w = 1;
+  int64_t best = full;
+  for (int cand = 2; cand <= 8; cand *= 2) {
+    if (full / cand < j || merge_lds_bytes(pl.vec, j, cand, cmp_size) > kMergeLdsLimit) break;
+    const int64_t cost = full / cand + (int64_t)(cand - 1) * j;
+    if (cost <= best) { best = cost; w = cand; }
+  }
   pl.waves = w;
 
   // Slabs: only when the grid would still be small and the runs are long.

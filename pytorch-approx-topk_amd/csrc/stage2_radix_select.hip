@@ -18,7 +18,15 @@ namespace {
 constexpr int kWave = 64;
 constexpr int kMaxWaves = 16;
 
+// Histogram counters are kept in kCopies private copies (lane % kCopies picks
+// one) so that the many candidates sharing a digit -- the top byte of a float
+// key is nearly constant among top-k candidates -- do not serialise on one LDS
+// address; the odd stride spreads equal digits of different copies over banks.
+constexpr int kCopies = 16;
+constexpr int kCopyStride = 257;
+
 struct SelectShared {
+  uint32_t copies[kCopies * kCopyStride];
   uint32_t hist[256];
   uint32_t wave_total[kMaxWaves];
   uint32_t digit;
@@ -71,6 +79,16 @@ __device__ inline void find_bin(SelectShared& sh, uint32_t need) {
   }
 }
 
+// hist[d] = sum of the private copies of bin d
+__device__ inline void fold_copies(SelectShared& sh, uint32_t tid, uint32_t nt) {
+  for (uint32_t d = tid; d < 256; d += nt) {
+    uint32_t total = 0;
+#pragma unroll
+    for (int c = 0; c < kCopies; ++c) total += sh.copies[c * kCopyStride + d];
+    sh.hist[d] = total;
+  }
+}
+
 template <typename E, bool KEYS_IN_LDS>
 __global__ __launch_bounds__(1024) void select_kernel(
     const typename E::raw_t* __restrict__ cand_values,
@@ -91,17 +109,20 @@ __global__ __launch_bounds__(1024) void select_kernel(
     for (uint32_t i = tid; i < k0; i += nt) keys[i] = E::key(cv[i]);
   }
   auto key_at = [&](uint32_t i) -> key_t { return KEYS_IN_LDS ? keys[i] : E::key(cv[i]); };
+  uint32_t* my_copy = &sh.copies[(tid % kCopies) * kCopyStride];  // this lane's histogram copy
 
   // ---- value select: T = key of the k-th best candidate --------------------
   key_t prefix = 0, mask = 0;
   uint32_t need = k;
   for (int shift = E::key_bits - 8; shift >= 0; shift -= 8) {
-    for (uint32_t i = tid; i < 256; i += nt) sh.hist[i] = 0;
+    for (uint32_t i = tid; i < kCopies * kCopyStride; i += nt) sh.copies[i] = 0;
     __syncthreads();
     for (uint32_t i = tid; i < k0; i += nt) {
       const key_t key = key_at(i);
-      if ((key & mask) == prefix) atomicAdd(&sh.hist[(uint32_t)(key >> shift) & 0xffu], 1u);
+      if ((key & mask) == prefix) atomicAdd(&my_copy[(uint32_t)(key >> shift) & 0xffu], 1u);
     }
+    __syncthreads();
+    fold_copies(sh, tid, nt);
     __syncthreads();
     find_bin<true>(sh, need);
     __syncthreads();
@@ -118,14 +139,16 @@ __global__ __launch_bounds__(1024) void select_kernel(
     uint64_t iprefix = 0, imask = 0;
     for (int shift = ((index_bits + 7) / 8 - 1) * 8; shift >= 0; shift -= 8) {
       __syncthreads();
-      for (uint32_t i = tid; i < 256; i += nt) sh.hist[i] = 0;
+      for (uint32_t i = tid; i < kCopies * kCopyStride; i += nt) sh.copies[i] = 0;
       __syncthreads();
       for (uint32_t i = tid; i < k0; i += nt) {
         if (key_at(i) == T) {
           const uint64_t idx = (uint64_t)ci[i];
-          if ((idx & imask) == iprefix) atomicAdd(&sh.hist[(uint32_t)(idx >> shift) & 0xffu], 1u);
+          if ((idx & imask) == iprefix) atomicAdd(&my_copy[(uint32_t)(idx >> shift) & 0xffu], 1u);
         }
       }
+      __syncthreads();
+      fold_copies(sh, tid, nt);
       __syncthreads();
       find_bin<false>(sh, need);
       __syncthreads();
