@@ -118,6 +118,12 @@ int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t
   if (k == k0)
     return atk_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws,
                       ws_bytes, stream);
+  {
+    bool handled = false;
+    const int rcf = atk::launch_fused_row(x, rows, n, row_stride, k0, j, k, layout, dtype, values,
+                                          indices, (hipStream_t)stream, &handled);
+    if (handled || rcf != ATK_OK) return rcf;
+  }
   const TopkPlan p = plan_topk(rows, n, k0, j, k, layout, dtype);
   if (!ws || ws_bytes < p.total) return ATK_ERR_WORKSPACE;
   unsigned char* base = static_cast<unsigned char*>(ws);

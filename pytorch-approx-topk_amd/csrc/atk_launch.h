@@ -22,6 +22,12 @@ int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_str
                          int j, int layout, int dtype, void* values, int64_t* indices, void* ws,
                          size_t ws_bytes, hipStream_t stream, bool* handled);
 
+// fused_row_plan.hip: both stages in one kernel, one workgroup per row, for
+// batches of many rows whose candidates fit in LDS.  `*handled` as above.
+int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                     int64_t k, int layout, int dtype, void* values, int64_t* indices,
+                     hipStream_t stream, bool* handled);
+
 // stage2_radix_select.hip: one workgroup per row.
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,

@@ -1,0 +1,180 @@
+// Both stages in one kernel, one workgroup per row.
+//
+// For batches of many moderate rows (a row's candidates fit in LDS) the
+// candidates never travel to HBM: the workgroup streams its row through the
+// same register queues as the streaming stage-1 kernel (stage1_stream.h),
+// parks the k0 candidates (raw value + sub-row number) in LDS, runs the
+// block-wide radix select of stage2_select.h over them and writes only the k
+// survivors.  HBM traffic is the input once plus the final k values and
+// indices per row; the two-kernel path additionally writes and re-reads
+// k0 * (sizeof(T) + 8) bytes per row.
+//
+// Work split inside the workgroup: the row's T column tiles (64*V columns each)
+// are shared out over the waves; with few tiles, `split` waves share a tile,
+// each scanning 1/split of the sub-rows, and fold through LDS as in the
+// streaming kernel.  Results are identical to atk_stage1 followed by
+// atk_select: same candidates in the same positions, same cut, same order.
+#pragma once
+
+#include "stage1_stream.h"
+#include "stage2_select.h"
+
+namespace atk {
+namespace fused {
+
+using stream::Cmp;
+using stream::Geom;
+using stream::kWave;
+
+// pos_t: uint16_t when every sub-row number fits, else uint32_t.
+template <typename E, int J, int V, int MAXW, typename pos_t>
+__global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
+    const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
+    int64_t* __restrict__ indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t k0, uint32_t k,
+    int index_bits) {
+  using raw_t = typename E::raw_t;
+  using key_t = typename E::key_t;
+  using C = Cmp<E>;
+  using cmp_t = typename C::cmp_t;
+  constexpr int kTileCols = kWave * V;
+  constexpr int U = J <= 2 ? 8 : 4;
+
+  extern __shared__ __align__(16) unsigned char dyn_lds[];
+  __shared__ select::Shared sh;
+  // candidates, then the hand-over area of the waves that share a tile
+  raw_t* cand_raw = reinterpret_cast<raw_t*>(dyn_lds);
+  const uint32_t pos_off = (k0 * (uint32_t)sizeof(raw_t) + 15u) & ~15u;
+  pos_t* cand_pos = reinterpret_cast<pos_t*>(dyn_lds + pos_off);
+  const uint32_t hand_off = (pos_off + k0 * (uint32_t)sizeof(pos_t) + 15u) & ~15u;
+  const uint32_t nwaves = blockDim.x / kWave;
+  const uint32_t helpers = nwaves - nwaves / split;  // waves that are not tile leaders
+  cmp_t* hand_q = reinterpret_cast<cmp_t*>(dyn_lds + hand_off);
+  uint32_t* hand_p = reinterpret_cast<uint32_t*>(dyn_lds + hand_off + (size_t)helpers * V * J * kWave * sizeof(cmp_t));
+
+  const uint32_t lane = threadIdx.x % kWave;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int64_t row = blockIdx.x;
+  const raw_t* xr = x + row * g.row_stride;
+
+  const uint32_t part = wave % split;            // which share of the sub-rows
+  const uint32_t group = wave / split;           // tile slot of this wave
+  const uint32_t groups = nwaves / split;        // tiles in flight per round
+  const uint32_t p0 = __builtin_amdgcn_readfirstlane((uint32_t)(((uint64_t)g.full_rows * part) / split));
+  const uint32_t p1 = __builtin_amdgcn_readfirstlane((uint32_t)(((uint64_t)g.full_rows * (part + 1)) / split));
+
+  bool any_nan = false;
+  for (uint32_t base = 0; base < tiles; base += groups) {  // same trip count for every wave
+    const uint32_t tile = base + group;
+    const bool has_tile = tile < tiles;
+    const int64_t col = (int64_t)tile * kTileCols + lane * V;
+    const bool live = has_tile && col < g.b;
+    cmp_t q[V][J];
+    uint32_t pos[V][J];
+    if (has_tile) {
+      uint64_t nan_mask = 0;
+      stream::scan_run<E, J, V, U>(xr, g, col, live, p0, p1, part == split - 1, q, pos, nan_mask);
+      any_nan |= C::has_nan && nan_mask != 0;
+    }
+    if (split > 1) {
+      if (has_tile && part > 0) {
+        const uint32_t slot = group * (split - 1) + (part - 1);
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+#pragma unroll
+          for (int s = 0; s < J; ++s) {
+            hand_q[((size_t)slot * V * J + v * J + s) * kWave + lane] = q[v][s];
+            hand_p[((size_t)slot * V * J + v * J + s) * kWave + lane] = pos[v][s];
+          }
+      }
+      __syncthreads();
+      if (has_tile && part == 0) {
+        // fold in sub-row order, each wave's entries best first: equal values keep the lowest index
+        for (uint32_t w = 0; w + 1 < split; ++w) {
+          const uint32_t slot = group * (split - 1) + w;
+#pragma unroll
+          for (int v = 0; v < V; ++v)
+#pragma unroll
+            for (int s = J - 1; s >= 0; --s)
+              stream::push<cmp_t, J, J>(q[v], pos[v], hand_q[((size_t)slot * V * J + v * J + s) * kWave + lane],
+                                        hand_p[((size_t)slot * V * J + v * J + s) * kWave + lane]);
+        }
+      }
+    }
+    if (live && part == 0) {
+#pragma unroll
+      for (int v = 0; v < V; ++v)
+#pragma unroll
+        for (int s = 0; s < J; ++s) {
+          cand_raw[(col + v) * J + s] = C::to_raw(q[v][s]);
+          cand_pos[(col + v) * J + s] = (pos_t)pos[v][s];
+        }
+    }
+    if (split > 1) __syncthreads();  // the hand-over area is reused by the next round
+  }
+
+  if (C::has_nan) {
+    if (__syncthreads_or(any_nan)) {
+      // a NaN was loaded somewhere in the row: redo stage 1 with exact order keys
+      for (int64_t c = threadIdx.x; c < g.b; c += blockDim.x) {
+        raw_t qv[J];
+        uint32_t qp[J];
+        int filled = 0;
+#pragma unroll
+        for (int s = 0; s < J; ++s) { qv[s] = 0; qp[s] = 0; }
+        for (uint32_t p = 0; p < g.full_rows; ++p) stream::push_exact<E, J>(qv, qp, filled, xr[(int64_t)p * g.b + c], p);
+        if (g.rem != 0) {
+          if (c < (int64_t)g.rem)
+            stream::push_exact<E, J>(qv, qp, filled, xr[(int64_t)g.full_rows * g.b + c], g.full_rows);
+          else if (g.pad_tail)
+            stream::push_exact<E, J>(qv, qp, filled, E::pad_raw, g.full_rows);
+        }
+#pragma unroll
+        for (int s = 0; s < J; ++s) { cand_raw[c * J + s] = qv[s]; cand_pos[c * J + s] = (pos_t)qp[s]; }
+      }
+    }
+  }
+  // (the select's first pass starts with a barrier, which also publishes the candidates)
+
+  auto key_at = [&](uint32_t i) -> key_t { return E::key(cand_raw[i]); };
+  auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)cand_pos[i] * (uint64_t)g.b + i / J; };
+  const select::Cut<key_t> cut =
+      select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
+
+  raw_t* ov = values + row * (int64_t)k;
+  int64_t* oi = indices + row * (int64_t)k;
+  select::compact(
+      sh, k0, k,
+      [&](uint32_t i) -> bool {
+        const key_t key = key_at(i);
+        if (key != cut.T) return key > cut.T;
+        return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
+      },
+      [&](uint32_t i, uint32_t o) {
+        ov[o] = cand_raw[i];
+        oi[o] = (int64_t)index_at(i);
+      });
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+struct Plan {
+  bool ok;
+  int vec;              // V
+  uint32_t full_rows, rem, pad_tail;
+  uint32_t tiles;       // column tiles per row
+  uint32_t split;       // waves sharing a tile
+  uint32_t waves;       // waves per workgroup
+  bool pos16;           // sub-row numbers fit 16 bits
+  int index_bits;
+  size_t lds_bytes;     // dynamic LDS
+};
+
+Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned);
+
+template <typename E>
+int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int64_t k0, int j,
+                 int64_t k, void* values, int64_t* indices, hipStream_t stream);
+
+}  // namespace fused
+}  // namespace atk

@@ -1,0 +1,8 @@
+// Fused one-workgroup-per-row kernel instantiated for one element type.
+#include "fused_row_launch.h"
+
+namespace atk {
+namespace fused {
+ATK_INSTANTIATE_FUSED(ATK_I16)
+}  // namespace fused
+}  // namespace atk

@@ -1,0 +1,59 @@
+// Launch code of the fused one-workgroup-per-row kernel for one element type.
+#pragma once
+
+#include "fused_row.h"
+
+namespace atk {
+namespace fused {
+
+template <typename E, int J, int V, int MAXW, typename pos_t>
+static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
+                      uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+  auto kern = fused_row_kernel<E, J, V, MAXW, pos_t>;
+  if (pl.lds_bytes > 48 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)pl.lds_bytes) != hipSuccess)
+      return ATK_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(kWave * pl.waves), pl.lds_bytes, stream, x, values,
+                     indices, g, pl.tiles, pl.split, k0, k, pl.index_bits);
+  return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+}
+
+template <typename E, int J>
+static int launch_j(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
+                    uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+  constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
+  if (pl.waves <= 4) {
+    return pl.pos16 ? launch_one<E, J, VF, 4, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
+                    : launch_one<E, J, VF, 4, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
+  }
+  return pl.pos16 ? launch_one<E, J, VF, 16, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
+                  : launch_one<E, J, VF, 16, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
+}
+
+template <typename E>
+int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int64_t k0, int j,
+                 int64_t k, void* values, int64_t* indices, hipStream_t stream) {
+  using raw_t = typename E::raw_t;
+  Geom g{};
+  g.row_stride = row_stride; g.b = k0 / j;
+  g.full_rows = pl.full_rows; g.rem = pl.rem; g.pad_tail = pl.pad_tail;
+  g.slabs = 1; g.slab_len = pl.full_rows; g.col_tiles = pl.tiles;
+  const raw_t* xs = static_cast<const raw_t*>(x);
+  raw_t* ov = static_cast<raw_t*>(values);
+  switch (j) {
+    case 1: return launch_j<E, 1>(pl, xs, rows, g, (uint32_t)k0, (uint32_t)k, ov, indices, stream);
+    case 2: return launch_j<E, 2>(pl, xs, rows, g, (uint32_t)k0, (uint32_t)k, ov, indices, stream);
+    case 3: return launch_j<E, 3>(pl, xs, rows, g, (uint32_t)k0, (uint32_t)k, ov, indices, stream);
+    case 4: return launch_j<E, 4>(pl, xs, rows, g, (uint32_t)k0, (uint32_t)k, ov, indices, stream);
+  }
+  return ATK_ERR_J;
+}
+
+#define ATK_INSTANTIATE_FUSED(DT)                                                                  \
+  template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int64_t, int,    \
+                                      int64_t, void*, int64_t*, hipStream_t);
+
+}  // namespace fused
+}  // namespace atk

@@ -1,0 +1,87 @@
+// Host-side planning and dispatch of the fused one-workgroup-per-row kernel.
+#include "fused_row.h"
+
+namespace atk {
+namespace fused {
+
+namespace {
+// Rows below which one workgroup per row would leave most of the 256 CUs idle.
+constexpr int64_t kMinRows = 128;
+// Dynamic LDS a workgroup may use (candidates + hand-over); the select's own
+// block adds about 18 KiB.
+constexpr size_t kLdsBudget = 64 * 1024;
+// Waves per workgroup: 16, or 4 for the element types whose lanes own 8 columns
+// (their queues need the register budget of a small workgroup).
+inline uint32_t max_waves(int vec) { return vec <= 4 ? 16u : 4u; }
+}  // namespace
+
+Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned) {
+  Plan pl{};
+  pl.ok = false;
+  if (layout != ATK_INTERLEAVED && layout != ATK_INTERLEAVED_PADDED) return pl;
+  if (!aligned || rows < kMinRows || rows > 0x7fffffffll) return pl;
+  if (k0 <= 0 || k <= 0 || k >= k0 || j < 1 || j > 4 || k0 % j) return pl;
+  const int es = elem_bytes(dtype);
+  if (!es) return pl;
+  const int64_t b = k0 / j;
+  const int64_t full = n / b;
+  if (full < j || full > 0x7fffffffll) return pl;
+  pl.vec = stream::full_vec(es);
+  if (b % pl.vec) return pl;
+  pl.full_rows = (uint32_t)full;
+  pl.rem = (uint32_t)(n - full * b);
+  pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
+  pl.pos16 = full + 1 <= 0xffff;
+  const int64_t bound = (full + 1) * b;  // indices are < this
+  pl.index_bits = 1;
+  while (pl.index_bits < 63 && (1ll << pl.index_bits) < bound) ++pl.index_bits;
+
+  const int64_t tile_cols = (int64_t)stream::kWave * pl.vec;
+  pl.tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
+  // Worth it only when parking the candidates in HBM would cost a good part of
+  // what reading the row costs: written and re-read k0*(es+8) bytes against n*es.
+  if ((size_t)k0 * (es + 8) * 4 < (size_t)n * es) return pl;
+  const size_t cand_bytes = (((size_t)k0 * es + 15) & ~(size_t)15) +
+                            (((size_t)k0 * (pl.pos16 ? 2 : 4) + 15) & ~(size_t)15);
+  if (cand_bytes > kLdsBudget) return pl;
+
+  // Waves sharing a tile: as many as keep each share at least max(j, 8)
+  // sub-rows long, the workgroup within 16 waves and the hand-over within LDS.
+  const int cmp_size = es > 4 ? 8 : 4;
+  const int64_t min_run = j > 8 ? j : 8;
+  const uint32_t kMaxWaves = max_waves(pl.vec);
+  uint32_t split = 1;
+  if (pl.tiles < kMaxWaves) {
+    for (uint32_t cand = 2; cand * pl.tiles <= kMaxWaves; cand *= 2) {
+      if (full / cand < min_run) break;
+      const size_t hand = (size_t)pl.tiles * (cand - 1) * pl.vec * j * stream::kWave * (cmp_size + 4);
+      if (cand_bytes + hand > kLdsBudget) break;
+      split = cand;
+    }
+  }
+  pl.split = split;
+  pl.waves = pl.tiles * split <= kMaxWaves ? pl.tiles * split : kMaxWaves;
+  const uint32_t helpers = pl.waves - pl.waves / split;
+  pl.lds_bytes = cand_bytes + (size_t)helpers * pl.vec * j * stream::kWave * (cmp_size + 4);
+  pl.ok = true;
+  return pl;
+}
+
+}  // namespace fused
+
+int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                     int64_t k, int layout, int dtype, void* values, int64_t* indices, hipStream_t stream,
+                     bool* handled) {
+  const int es = elem_bytes(dtype);
+  const int vf = es ? stream::full_vec(es) : 1;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && (row_stride % vf == 0);
+  const fused::Plan pl = fused::make_plan(rows, n, k0, j, k, layout, dtype, aligned);
+  *handled = pl.ok;
+  if (!pl.ok) return ATK_OK;
+  int rc = ATK_ERR_DTYPE;
+  ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
+                   rc = fused::launch_typed<E>(pl, x, rows, row_stride, k0, j, k, values, indices, stream));
+  return rc;
+}
+
+}  // namespace atk

@@ -253,40 +253,20 @@ __device__ inline void exact_columns(const typename E::raw_t* __restrict__ xr, c
   emit<E, J, V>(g, out, row, slab, col, val, pos);
 }
 
-// E: element traits; J: entries kept per bucket; V: columns per lane; W: waves
-// per workgroup, sharing one column tile and splitting its sub-rows; U: loads
-// kept in flight per lane.
-template <typename E, int J, int V, int W, int U>
-__global__ __launch_bounds__(kWave * W) void stream_kernel(
-    const typename E::raw_t* __restrict__ x, const Sink<typename E::raw_t> out, const Geom g) {
+// One wave's scan: the top J of sub-rows [p0, p1) (p1 - p0 >= J) for this lane's V
+// columns starting at `col`, plus the row's partial sub-row when `with_rem`.
+// `xr` is the row; lanes that are not `live` load column 0 and are ignored by
+// the caller.  U loads stay in flight per lane.  Sets bits in `nan_mask`
+// (wave-uniform) for lanes that loaded a NaN; the queues are meaningless then.
+template <typename E, int J, int V, int U>
+__device__ inline void scan_run(const typename E::raw_t* __restrict__ xr, const Geom& g, int64_t col,
+                                bool live, uint32_t p0, uint32_t p1, bool with_rem,
+                                typename Cmp<E>::cmp_t (&q)[V][J], uint32_t (&pos)[V][J],
+                                uint64_t& nan_mask) {
   using raw_t = typename E::raw_t;
   using C = Cmp<E>;
   using cmp_t = typename C::cmp_t;
   static_assert(U >= J, "the first U loads must cover the J sub-rows that fill the queues");
-  constexpr int kTileCols = kWave * V;
-
-  const uint32_t lane = threadIdx.x % kWave;
-  // Everything that decides control flow is wave-uniform; say so, so that it
-  // lives in scalar registers.
-  const uint32_t wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) : 0;
-  uint32_t blk = blockIdx.x;
-  const uint32_t col_tile = __builtin_amdgcn_readfirstlane(blk % g.col_tiles);
-  blk /= g.col_tiles;
-  const uint32_t slab = __builtin_amdgcn_readfirstlane(blk % g.slabs);
-  const int64_t row = __builtin_amdgcn_readfirstlane(blk / g.slabs);
-
-  const int64_t col = (int64_t)col_tile * kTileCols + lane * V;
-  const bool live = col < g.b;  // b is a multiple of V whenever V > 1
-
-  // sub-rows of this slab [s0, s1), then of this wave [p0, p1)
-  const uint32_t s0 = slab * g.slab_len;
-  const uint32_t s1 = (slab + 1 == g.slabs) ? g.full_rows : s0 + g.slab_len;
-  const uint32_t p0 = __builtin_amdgcn_readfirstlane(s0 + (uint32_t)(((uint64_t)(s1 - s0) * wave) / W));
-  const uint32_t p1 = __builtin_amdgcn_readfirstlane(s0 + (uint32_t)(((uint64_t)(s1 - s0) * (wave + 1)) / W));
-  const bool last_slab = slab + 1 == g.slabs;
-  const bool last_run = last_slab && wave == W - 1;
-
-  const raw_t* xr = x + row * g.row_stride;
   // `next` walks down this lane's columns one sub-row per load
   const raw_t* next = xr + (live ? col : 0) + (int64_t)p0 * g.b;
   auto load_next = [&]() {
@@ -294,11 +274,6 @@ __global__ __launch_bounds__(kWave * W) void stream_kernel(
     next += g.b;
     return pk;
   };
-
-  cmp_t q[V][J];
-  uint32_t pos[V][J];
-  uint64_t nan_mask = 0;  // lanes that saw a NaN; wave-uniform
-
   auto take = [&](const Pack<raw_t, V>& pk, uint32_t p, auto filled_tag) {
     constexpr int FILLED = decltype(filled_tag)::value;
     cmp_t c[V];
@@ -313,8 +288,8 @@ __global__ __launch_bounds__(kWave * W) void stream_kernel(
     for (int v = 0; v < V; ++v) push<cmp_t, J, FILLED>(q[v], pos[v], c[v], p);
   };
 
-  // U loads stay in flight.  Slot u of `buf` holds sub-row p + u; consuming it
-  // frees the slot for sub-row p + U + u.  `ld` is the next sub-row to load.
+  // Slot u of `buf` holds sub-row p + u; consuming it frees the slot for
+  // sub-row p + U + u.  `ld` is the next sub-row to load.
   Pack<raw_t, V> buf[U];
   uint32_t ld = p0;
 #pragma unroll
@@ -322,7 +297,7 @@ __global__ __launch_bounds__(kWave * W) void stream_kernel(
     if (ld < p1) { buf[u] = load_next(); ++ld; }
   }
   uint32_t p = p0;
-  // first group: also fills the queues (the run has at least J sub-rows)
+  // first group: also fills the queues
   static_for<U>([&](auto uc) {
     constexpr int u = decltype(uc)::value;
     if (p0 + u < p1) {
@@ -356,7 +331,7 @@ __global__ __launch_bounds__(kWave * W) void stream_kernel(
   }
   // the partial sub-row: column c has one more element when c < rem
   // (with a padded row the other columns see the pad value there)
-  if (last_run && g.rem != 0) {
+  if (with_rem && g.rem != 0) {
 #pragma unroll
     for (int v = 0; v < V; ++v) {
       const bool real = col + v < (int64_t)g.rem;
@@ -367,6 +342,44 @@ __global__ __launch_bounds__(kWave * W) void stream_kernel(
       }
     }
   }
+}
+
+// E: element traits; J: entries kept per bucket; V: columns per lane; W: waves
+// per workgroup, sharing one column tile and splitting its sub-rows; U: loads
+// kept in flight per lane.
+template <typename E, int J, int V, int W, int U>
+__global__ __launch_bounds__(kWave * W) void stream_kernel(
+    const typename E::raw_t* __restrict__ x, const Sink<typename E::raw_t> out, const Geom g) {
+  using raw_t = typename E::raw_t;
+  using C = Cmp<E>;
+  using cmp_t = typename C::cmp_t;
+  constexpr int kTileCols = kWave * V;
+
+  const uint32_t lane = threadIdx.x % kWave;
+  // Everything that decides control flow is wave-uniform; say so, so that it
+  // lives in scalar registers.
+  const uint32_t wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) : 0;
+  uint32_t blk = blockIdx.x;
+  const uint32_t col_tile = __builtin_amdgcn_readfirstlane(blk % g.col_tiles);
+  blk /= g.col_tiles;
+  const uint32_t slab = __builtin_amdgcn_readfirstlane(blk % g.slabs);
+  const int64_t row = __builtin_amdgcn_readfirstlane(blk / g.slabs);
+
+  const int64_t col = (int64_t)col_tile * kTileCols + lane * V;
+  const bool live = col < g.b;  // b is a multiple of V whenever V > 1
+
+  // sub-rows of this slab [s0, s1), then of this wave [p0, p1)
+  const uint32_t s0 = slab * g.slab_len;
+  const uint32_t s1 = (slab + 1 == g.slabs) ? g.full_rows : s0 + g.slab_len;
+  const uint32_t p0 = __builtin_amdgcn_readfirstlane(s0 + (uint32_t)(((uint64_t)(s1 - s0) * wave) / W));
+  const uint32_t p1 = __builtin_amdgcn_readfirstlane(s0 + (uint32_t)(((uint64_t)(s1 - s0) * (wave + 1)) / W));
+  const bool last_slab = slab + 1 == g.slabs;
+
+  const raw_t* xr = x + row * g.row_stride;
+  cmp_t q[V][J];
+  uint32_t pos[V][J];
+  uint64_t nan_mask = 0;
+  scan_run<E, J, V, U>(xr, g, col, live, p0, p1, last_slab && wave == W - 1, q, pos, nan_mask);
 
   bool any_nan = C::has_nan && nan_mask != 0;
   if constexpr (W > 1) {

@@ -14,7 +14,7 @@ static int launch_one(const Plan& pl, const typename E::raw_t* x, const Sink<typ
   if (groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   // combinations the planner never picks are not compiled
   if constexpr (merge_lds_bytes(V, J, W, sizeof(typename Cmp<E>::cmp_t)) <= kMergeLdsLimit) {
-    hipLaunchKernelGGL((stream_kernel<E, J, V, W, 8>), dim3((unsigned)groups), dim3(kWave * W), 0,
+    hipLaunchKernelGGL((stream_kernel<E, J, V, W, (J <= 2 ? 8 : 4)>), dim3((unsigned)groups), dim3(kWave * W), 0,
                        stream, x, out, g);
     return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
   } else {

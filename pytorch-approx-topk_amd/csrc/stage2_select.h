@@ -1,0 +1,188 @@
+// Block-wide exact top-k selection over candidates held by one workgroup.
+//
+// An MSB-first radix select with 8-bit digits finds the order key T of the k-th
+// best candidate and how many of the candidates with key == T belong to the
+// result; when only part of that tie group belongs, a second radix select over
+// the candidates' original indices finds the cut so that the lowest indices
+// win.  Survivors are then emitted in increasing candidate position with
+// wave-level ballot/mbcnt compaction.  Candidates are reached through
+// accessors, so the same code serves keys staged in LDS, keys re-read from
+// global memory, and candidates that never left the workgroup.
+//
+// Every function here must be called by all threads of the workgroup.
+#pragma once
+
+#include "atk_device.h"
+
+namespace atk {
+namespace select {
+
+constexpr int kWave = 64;
+constexpr int kMaxWaves = 16;
+
+// Histogram counters are kept in kCopies private copies (lane % kCopies picks
+// one) so that the many candidates sharing a digit -- the top byte of a float
+// key is nearly constant among top-k candidates -- do not serialise on one LDS
+// address; the odd stride spreads equal digits of different copies over banks.
+constexpr int kCopies = 16;
+constexpr int kCopyStride = 257;
+
+struct Shared {
+  uint32_t copies[kCopies * kCopyStride];
+  uint32_t hist[256];
+  uint32_t wave_total[kMaxWaves];
+  uint32_t digit;
+  uint32_t need;
+  uint32_t bin_count;
+};
+
+__device__ inline uint32_t lane_id() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// Number of set bits of `m` below this lane.
+__device__ inline uint32_t rank_in(uint64_t m) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                   __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+}
+
+// hist[d] = sum of the private copies of bin d
+__device__ inline void fold_copies(Shared& sh) {
+  for (uint32_t d = threadIdx.x; d < 256; d += blockDim.x) {
+    uint32_t total = 0;
+#pragma unroll
+    for (int c = 0; c < kCopies; ++c) total += sh.copies[c * kCopyStride + d];
+    sh.hist[d] = total;
+  }
+}
+
+// Wave 0 scans the 256-bin histogram for the bin holding the `need`-th element,
+// counting from the top bin (FROM_TOP) or from the bottom bin, and publishes
+// the bin, the rank left within it and the bin's population.
+template <bool FROM_TOP>
+__device__ inline void find_bin(Shared& sh, uint32_t need) {
+  if (threadIdx.x < kWave) {
+    const uint32_t lane = threadIdx.x;
+    // Lane l owns bins 4l..4l+3.
+    uint32_t h[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h[i] = sh.hist[4 * lane + i];
+    const uint32_t mine = h[0] + h[1] + h[2] + h[3];
+    // Inclusive scan over lanes in scan order (descending lanes when FROM_TOP).
+    uint32_t incl = mine;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const uint32_t other = FROM_TOP ? __shfl_down(incl, d, kWave) : __shfl_up(incl, d, kWave);
+      const bool has = FROM_TOP ? (lane + d < kWave) : (lane >= (uint32_t)d);
+      if (has) incl += other;
+    }
+    uint32_t before = incl - mine;  // population of all bins scanned before this lane's
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int bin = FROM_TOP ? 3 - i : i;
+      const uint32_t c = h[bin];
+      if (before < need && need <= before + c) {
+        sh.digit = 4 * lane + bin;
+        sh.need = need - before;
+        sh.bin_count = c;
+      }
+      before += c;
+    }
+  }
+}
+
+// One radix pass: histogram digit `shift` of the values `digit_source(i)` over
+// the candidates with `participates(i)`, then locate the bin of rank `need`.
+template <bool FROM_TOP, typename Participates>
+__device__ inline void radix_pass(Shared& sh, uint32_t k0, uint32_t need, Participates digit_or_skip) {
+  const uint32_t tid = threadIdx.x, nt = blockDim.x;
+  uint32_t* my_copy = &sh.copies[(tid % kCopies) * kCopyStride];
+  __syncthreads();
+  for (uint32_t i = tid; i < kCopies * kCopyStride; i += nt) sh.copies[i] = 0;
+  __syncthreads();
+  for (uint32_t i = tid; i < k0; i += nt) {
+    const int d = digit_or_skip(i);  // 0..255, or -1 when candidate i is out of the race
+    if (d >= 0) atomicAdd(&my_copy[d], 1u);
+  }
+  __syncthreads();
+  fold_copies(sh);
+  __syncthreads();
+  find_bin<FROM_TOP>(sh, need);
+  __syncthreads();
+}
+
+// The cut: candidate i survives iff key(i) > T, or key(i) == T and index(i) <= index_cut.
+template <typename key_t> struct Cut {
+  key_t T;
+  uint64_t index_cut;  // ~0: every tie survives
+};
+
+// key_at(i): order key of candidate i; index_at(i): its original index (only
+// read for candidates tied at T, and only when the tie group is cut).
+template <typename key_t, int KEY_BITS, typename KeyAt, typename IndexAt>
+__device__ inline Cut<key_t> find_cut(Shared& sh, uint32_t k0, uint32_t k, int index_bits, KeyAt key_at,
+                                      IndexAt index_at) {
+  key_t prefix = 0, mask = 0;
+  uint32_t need = k;
+  for (int shift = KEY_BITS - 8; shift >= 0; shift -= 8) {
+    radix_pass<true>(sh, k0, need, [&](uint32_t i) -> int {
+      const key_t key = key_at(i);
+      return (key & mask) == prefix ? (int)((uint32_t)(key >> shift) & 0xffu) : -1;
+    });
+    prefix |= (key_t)sh.digit << shift;
+    mask |= (key_t)0xff << shift;
+    need = sh.need;
+  }
+  Cut<key_t> cut{prefix, ~0ull};
+  const uint32_t ties = sh.bin_count;  // candidates with key == T
+  if (need < ties) {                   // uniform over the workgroup
+    uint64_t iprefix = 0, imask = 0;
+    for (int shift = ((index_bits + 7) / 8 - 1) * 8; shift >= 0; shift -= 8) {
+      radix_pass<false>(sh, k0, need, [&](uint32_t i) -> int {
+        if (key_at(i) != cut.T) return -1;
+        const uint64_t idx = index_at(i);
+        return (idx & imask) == iprefix ? (int)((uint32_t)(idx >> shift) & 0xffu) : -1;
+      });
+      iprefix |= (uint64_t)sh.digit << shift;
+      imask |= (uint64_t)0xff << shift;
+      need = sh.need;
+    }
+    cut.index_cut = iprefix;
+  }
+  return cut;
+}
+
+// Stable compaction: wave w owns a contiguous run of candidates; emit(i, o)
+// is called for every surviving candidate i with its output slot o < k.
+template <typename Survives, typename Emit>
+__device__ inline void compact(Shared& sh, uint32_t k0, uint32_t k, Survives survives, Emit emit) {
+  const uint32_t tid = threadIdx.x, nt = blockDim.x;
+  const uint32_t waves = nt / kWave, wave = tid / kWave, lane = lane_id();
+  uint32_t per_wave = (k0 + waves - 1) / waves;
+  per_wave = (per_wave + kWave - 1) / kWave * kWave;
+  const uint32_t lo = min(wave * per_wave, k0), hi = min(lo + per_wave, k0);
+  uint32_t mine = 0;
+  for (uint32_t base = lo; base < hi; base += kWave) {
+    const uint32_t i = base + lane;
+    const bool sel = i < hi && survives(i);
+    mine += (uint32_t)__popcll(__ballot(sel));
+  }
+  __syncthreads();
+  if (lane == 0) sh.wave_total[wave] = mine;
+  __syncthreads();
+  uint32_t out = 0;
+  for (uint32_t w = 0; w < wave; ++w) out += sh.wave_total[w];
+  for (uint32_t base = lo; base < hi; base += kWave) {
+    const uint32_t i = base + lane;
+    const bool sel = i < hi && survives(i);
+    const uint64_t m = __ballot(sel);
+    if (sel) {
+      const uint32_t o = out + rank_in(m);
+      if (o < k) emit(i, o);
+    }
+    out += (uint32_t)__popcll(m);
+  }
+}
+
+}  // namespace select
+}  // namespace atk

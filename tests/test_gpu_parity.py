@@ -250,3 +250,62 @@ def test_torch_compile_fullgraph(dtype, interleaved):
     ev, ei = topk(**kw)
     cv, ci = compiled(**kw)
     assert torch.equal(ev, cv) and torch.equal(ei, ci)
+
+
+# ---- shapes that take the fused one-workgroup-per-row kernel (many rows, k_mult > 1) ----
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("j,k_mult", [(1, 2), (2, 4), (3, 2), (4, 4)])
+def test_fused_rows_all_dtypes_with_ties(dtype, j, k_mult):
+    g = torch.Generator().manual_seed(11 + j)
+    shape = (130, 2048)
+    if dtype.is_floating_point:
+        x = torch.randint(-9, 10, shape, generator=g).to(dtype) / 4
+    elif dtype == torch.uint8:
+        x = torch.randint(0, 19, shape, generator=g).to(dtype)
+    else:
+        x = torch.randint(-9, 10, shape, generator=g).to(dtype)
+    _check(x, 48, -1, j=j, k_mult=k_mult)
+
+
+@pytest.mark.parametrize("n,k,j,k_mult", [
+    (4096, 64, 1, 8),      # two tiles, long columns: waves share a tile
+    (4100, 64, 2, 4),      # partial last sub-row
+    (32768, 2048, 4, 4),   # the sparse-attention shape, fp32
+    (16384, 1024, 2, 8),   # 4096 columns: more tiles than waves
+    (1000, 100, 4, 2),     # bucket count not a multiple of the vector width -> general path
+    (777, 12, 3, 5),
+])
+def test_fused_rows_shapes(n, k, j, k_mult):
+    _check(cpu_randn((136, n), n + k), k, -1, j=j, k_mult=k_mult)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+def test_fused_rows_special_values(dtype):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((140, 4096), generator=g).to(dtype)
+    specials = torch.tensor([float("nan"), float("inf"), -float("inf"), 0.0, -0.0]).to(dtype)
+    for r in range(0, 140, 3):     # every third row holds special values, NaN included
+        sel = torch.randint(0, 4096, (300,), generator=g)
+        x[r, sel] = specials[torch.randint(0, 5, (300,), generator=g)]
+    for j, km in [(1, 4), (2, 2), (4, 2)]:
+        _check(x, 256, -1, j=j, k_mult=km)
+
+
+def test_fused_rows_all_equal_cut_ties_by_index():
+    x = torch.zeros(129, 4096)
+    x[1::2] = 1.5
+    for j, km in [(1, 2), (2, 4), (4, 8)]:
+        _check(x, 128, -1, j=j, k_mult=km)
+
+
+def test_fused_config3_and_config4_full_shapes():
+    x3 = (cpu_randn((1024, 32768), 1003) / 128 ** 0.5).half()
+    v, i = _run(x3, 2048, -1, j=4, k_mult=4)
+    ev, ei = oracle_topk(x3[:96], 2048, -1, j=4, k_mult=4)
+    assert_same(v[:96], i[:96], ev, ei, "C3 first 96 rows")
+    assert torch.equal(x3.gather(-1, i.cpu()).view(torch.int16), v.cpu().view(torch.int16))
+    x4 = cpu_randn((256, 131072), 1004)
+    v, i = _run(x4, 64, -1, j=1, k_mult=8)
+    ev, ei = oracle_topk(x4, 64, -1, j=1, k_mult=8)
+    assert_same(v, i, ev, ei, "C4")
