@@ -26,18 +26,18 @@ using stream::Cmp;
 using stream::Geom;
 using stream::kWave;
 
-// pos_t: uint16_t when every sub-row number fits, else uint32_t.
-template <typename E, int J, int V, int MAXW, typename pos_t>
+// pos_t: uint16_t when every sub-row number fits, else uint32_t.  PACKED: packed
+// 16-bit queues (stage1_stream.h).
+template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
 __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
     int64_t* __restrict__ indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t k0, uint32_t k,
     int index_bits) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
-  using C = Cmp<E>;
-  using cmp_t = typename C::cmp_t;
+  using Queue = stream::QueueFor<E, J, V, PACKED>;
   constexpr int kTileCols = kWave * V;
-  constexpr int U = J <= 2 ? 8 : 4;
+  constexpr int U = PACKED ? (V * J <= 8 ? 8 : 4) : (J <= 2 ? 8 : 4);
 
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   __shared__ select::Shared sh;
@@ -47,9 +47,7 @@ __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
   pos_t* cand_pos = reinterpret_cast<pos_t*>(dyn_lds + pos_off);
   const uint32_t hand_off = (pos_off + k0 * (uint32_t)sizeof(pos_t) + 15u) & ~15u;
   const uint32_t nwaves = blockDim.x / kWave;
-  const uint32_t helpers = nwaves - nwaves / split;  // waves that are not tile leaders
-  cmp_t* hand_q = reinterpret_cast<cmp_t*>(dyn_lds + hand_off);
-  uint32_t* hand_p = reinterpret_cast<uint32_t*>(dyn_lds + hand_off + (size_t)helpers * V * J * kWave * sizeof(cmp_t));
+  unsigned char* hand = dyn_lds + hand_off;  // one Queue::kHandBytes area per wave that is not a tile leader
 
   const uint32_t lane = threadIdx.x % kWave;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -68,69 +66,46 @@ __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
     const bool has_tile = tile < tiles;
     const int64_t col = (int64_t)tile * kTileCols + lane * V;
     const bool live = has_tile && col < g.b;
-    cmp_t q[V][J];
-    uint32_t pos[V][J];
+    Queue queue;
     if (has_tile) {
-      uint64_t nan_mask = 0;
-      stream::scan_run<E, J, V, U>(xr, g, col, live, p0, p1, part == split - 1, q, pos, nan_mask);
-      any_nan |= C::has_nan && nan_mask != 0;
+      stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, part == split - 1, queue);
+      any_nan |= queue.poisoned();
     }
     if (split > 1) {
-      if (has_tile && part > 0) {
-        const uint32_t slot = group * (split - 1) + (part - 1);
-#pragma unroll
-        for (int v = 0; v < V; ++v)
-#pragma unroll
-          for (int s = 0; s < J; ++s) {
-            hand_q[((size_t)slot * V * J + v * J + s) * kWave + lane] = q[v][s];
-            hand_p[((size_t)slot * V * J + v * J + s) * kWave + lane] = pos[v][s];
-          }
-      }
+      if (has_tile && part > 0)
+        queue.hand_over(hand + (size_t)(group * (split - 1) + (part - 1)) * Queue::kHandBytes, lane);
       __syncthreads();
       if (has_tile && part == 0) {
-        // fold in sub-row order, each wave's entries best first: equal values keep the lowest index
-        for (uint32_t w = 0; w + 1 < split; ++w) {
-          const uint32_t slot = group * (split - 1) + w;
-#pragma unroll
-          for (int v = 0; v < V; ++v)
-#pragma unroll
-            for (int s = J - 1; s >= 0; --s)
-              stream::push<cmp_t, J, J>(q[v], pos[v], hand_q[((size_t)slot * V * J + v * J + s) * kWave + lane],
-                                        hand_p[((size_t)slot * V * J + v * J + s) * kWave + lane]);
-        }
+        for (uint32_t w = 0; w + 1 < split; ++w)
+          queue.fold_in(hand + (size_t)(group * (split - 1) + w) * Queue::kHandBytes, lane);
       }
     }
     if (live && part == 0) {
-#pragma unroll
-      for (int v = 0; v < V; ++v)
-#pragma unroll
-        for (int s = 0; s < J; ++s) {
-          cand_raw[(col + v) * J + s] = C::to_raw(q[v][s]);
-          cand_pos[(col + v) * J + s] = (pos_t)pos[v][s];
-        }
+      queue.fix_zeros(xr, g.b, col);
+      ATK_STATIC_FOR(e, V * J) {
+        cand_raw[col * J + e] = queue.template raw<e / J, e % J>();
+        cand_pos[col * J + e] = (pos_t)queue.template position<e / J, e % J>();
+      } ATK_STATIC_END;
     }
     if (split > 1) __syncthreads();  // the hand-over area is reused by the next round
   }
 
-  if (C::has_nan) {
-    if (__syncthreads_or(any_nan)) {
-      // a NaN was loaded somewhere in the row: redo stage 1 with exact order keys
-      for (int64_t c = threadIdx.x; c < g.b; c += blockDim.x) {
-        raw_t qv[J];
-        uint32_t qp[J];
-        int filled = 0;
-#pragma unroll
-        for (int s = 0; s < J; ++s) { qv[s] = 0; qp[s] = 0; }
-        for (uint32_t p = 0; p < g.full_rows; ++p) stream::push_exact<E, J>(qv, qp, filled, xr[(int64_t)p * g.b + c], p);
-        if (g.rem != 0) {
-          if (c < (int64_t)g.rem)
-            stream::push_exact<E, J>(qv, qp, filled, xr[(int64_t)g.full_rows * g.b + c], g.full_rows);
-          else if (g.pad_tail)
-            stream::push_exact<E, J>(qv, qp, filled, E::pad_raw, g.full_rows);
-        }
-#pragma unroll
-        for (int s = 0; s < J; ++s) { cand_raw[c * J + s] = qv[s]; cand_pos[c * J + s] = (pos_t)qp[s]; }
+  if (__syncthreads_or(any_nan)) {
+    // a value the fast queues cannot order (NaN; -0.0 for packed queues) was
+    // loaded somewhere in the row: redo stage 1 with exact order keys
+    for (int64_t c = threadIdx.x; c < g.b; c += blockDim.x) {
+      raw_t qv[J];
+      uint32_t qp[J];
+      stream::clear_exact<E, J>(qv, qp);
+      for (uint32_t p = 0; p < g.full_rows; ++p) stream::push_exact<E, J>(qv, qp, xr[(int64_t)p * g.b + c], p);
+      if (g.rem != 0) {
+        if (c < (int64_t)g.rem)
+          stream::push_exact<E, J>(qv, qp, xr[(int64_t)g.full_rows * g.b + c], g.full_rows);
+        else if (g.pad_tail)
+          stream::push_exact<E, J>(qv, qp, E::pad_raw, g.full_rows);
       }
+#pragma unroll
+      for (int s = 0; s < J; ++s) { cand_raw[c * J + s] = qv[s]; cand_pos[c * J + s] = (pos_t)qp[s]; }
     }
   }
   // (the select's first pass starts with a barrier, which also publishes the candidates)
@@ -166,6 +141,7 @@ struct Plan {
   uint32_t split;       // waves sharing a tile
   uint32_t waves;       // waves per workgroup
   bool pos16;           // sub-row numbers fit 16 bits
+  bool packed;          // packed 16-bit queues
   int index_bits;
   size_t lds_bytes;     // dynamic LDS
 };

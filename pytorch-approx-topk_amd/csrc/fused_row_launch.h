@@ -6,10 +6,10 @@
 namespace atk {
 namespace fused {
 
-template <typename E, int J, int V, int MAXW, typename pos_t>
-static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
-                      uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
-  auto kern = fused_row_kernel<E, J, V, MAXW, pos_t>;
+template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
+static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
+                         uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+  auto kern = fused_row_kernel<E, J, V, MAXW, pos_t, PACKED>;
   if (pl.lds_bytes > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)pl.lds_bytes) != hipSuccess)
@@ -18,6 +18,16 @@ static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, 
   hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(kWave * pl.waves), pl.lds_bytes, stream, x, values,
                      indices, g, pl.tiles, pl.split, k0, k, pl.index_bits);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+}
+
+template <typename E, int J, int V, int MAXW, typename pos_t>
+static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
+                      uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+  if constexpr (stream::PackedKey<E>::available && sizeof(pos_t) == 2) {
+    // packed queues need every sub-row number to fit 16 bits, as pos_t == uint16_t does
+    if (pl.packed) return launch_packed<E, J, V, MAXW, pos_t, true>(pl, x, rows, g, k0, k, values, indices, stream);
+  }
+  return launch_packed<E, J, V, MAXW, pos_t, false>(pl, x, rows, g, k0, k, values, indices, stream);
 }
 
 template <typename E, int J>

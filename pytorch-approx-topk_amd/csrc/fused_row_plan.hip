@@ -32,6 +32,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   pl.rem = (uint32_t)(n - full * b);
   pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
   pl.pos16 = full + 1 <= 0xffff;
+  pl.packed = (dtype == ATK_F16 || dtype == ATK_BF16 || dtype == ATK_I16) && full <= stream::kPackedMaxSubRow;
   const int64_t bound = (full + 1) * b;  // indices are < this
   pl.index_bits = 1;
   while (pl.index_bits < 63 && (1ll << pl.index_bits) < bound) ++pl.index_bits;

@@ -7,16 +7,34 @@
 namespace atk {
 namespace stream {
 
+template <typename E, int J, int V, int W, int RUN>
+static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
+                      const Geom& g, dim3 grid, hipStream_t stream) {
+  constexpr int U = J <= 2 ? 8 : 4;
+  if constexpr (PackedKey<E>::available) {
+    if (pl.packed) {
+      hipLaunchKernelGGL((stream_kernel<E, J, V, W, (V * J <= 8 ? 8 : 4), RUN, true>), grid, dim3(kWave * W), 0,
+                         stream, x, out, g);
+      return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+    }
+  }
+  hipLaunchKernelGGL((stream_kernel<E, J, V, W, U, RUN, false>), grid, dim3(kWave * W), 0, stream, x, out, g);
+  return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+}
+
 template <typename E, int J, int V, int W>
 static int launch_one(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
                       const Geom& g, int64_t rows, hipStream_t stream) {
   const int64_t groups = rows * (int64_t)pl.slabs * pl.col_tiles;
   if (groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
+  const dim3 grid((unsigned)groups);
   // combinations the planner never picks are not compiled
   if constexpr (merge_lds_bytes(V, J, W, sizeof(typename Cmp<E>::cmp_t)) <= kMergeLdsLimit) {
-    hipLaunchKernelGGL((stream_kernel<E, J, V, W, (J <= 2 ? 8 : 4)>), dim3((unsigned)groups), dim3(kWave * W), 0,
-                       stream, x, out, g);
-    return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+    if constexpr (V > 1) {  // exact short runs exist for the vector kernels only
+      if (pl.run == 4) return launch_run<E, J, V, W, 4>(pl, x, out, g, grid, stream);
+      if (pl.run == 8) return launch_run<E, J, V, W, 8>(pl, x, out, g, grid, stream);
+    }
+    return launch_run<E, J, V, W, 0>(pl, x, out, g, grid, stream);
   } else {
     (void)x; (void)out; (void)g; (void)stream;
     return ATK_ERR_ARG;

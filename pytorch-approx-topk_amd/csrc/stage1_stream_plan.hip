@@ -25,12 +25,13 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   if (!es) return pl;
   const int64_t b = k0 / j;
   const int64_t full = n / b;
-  if (full < j || full > 0xffffffffll || b > 0x7fffffffll) return pl;
+  if (full < j || full > 0xfffffffell || b > 0x7fffffffll) return pl;
   pl.full_rows = (uint32_t)full;
   pl.rem = (uint32_t)(n - full * b);
   pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
   const int vf = full_vec(es);
   pl.vec = (aligned && b % vf == 0) ? vf : 1;
+  pl.packed = (dtype == ATK_F16 || dtype == ATK_BF16 || dtype == ATK_I16) && full <= kPackedMaxSubRow;
 
   const int64_t tile_cols = (int64_t)kWave * pl.vec;
   pl.col_tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
@@ -68,6 +69,12 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
     if (const char* s = getenv("ATK_TUNE_SLABS")) pl.slabs = (uint32_t)atoi(s);
   }
   pl.slab_len = (uint32_t)(full / pl.slabs);
+  // every wave scans exactly 4 or 8 sub-rows: straight-line kernels exist for that
+  pl.run = 0;
+  if (pl.vec > 1 && pl.slabs == 1 && full % pl.waves == 0) {
+    const int64_t run = full / pl.waves;
+    if ((run == 4 || run == 8) && run >= j) pl.run = (int)run;
+  }
   if (pl.slabs > 1) {
     const size_t entries = (size_t)rows * pl.slabs * (size_t)k0;
     pl.part_values_off = 0;

@@ -36,18 +36,18 @@ struct Shared {
   uint32_t bin_count;
 };
 
-__device__ inline uint32_t lane_id() {
+__device__ __forceinline__ uint32_t lane_id() {
   return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }
 
 // Number of set bits of `m` below this lane.
-__device__ inline uint32_t rank_in(uint64_t m) {
+__device__ __forceinline__ uint32_t rank_in(uint64_t m) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
                                    __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
 }
 
 // hist[d] = sum of the private copies of bin d
-__device__ inline void fold_copies(Shared& sh) {
+__device__ __forceinline__ void fold_copies(Shared& sh) {
   for (uint32_t d = threadIdx.x; d < 256; d += blockDim.x) {
     uint32_t total = 0;
 #pragma unroll
@@ -60,7 +60,7 @@ __device__ inline void fold_copies(Shared& sh) {
 // counting from the top bin (FROM_TOP) or from the bottom bin, and publishes
 // the bin, the rank left within it and the bin's population.
 template <bool FROM_TOP>
-__device__ inline void find_bin(Shared& sh, uint32_t need) {
+__device__ __forceinline__ void find_bin(Shared& sh, uint32_t need) {
   if (threadIdx.x < kWave) {
     const uint32_t lane = threadIdx.x;
     // Lane l owns bins 4l..4l+3.
@@ -94,7 +94,7 @@ __device__ inline void find_bin(Shared& sh, uint32_t need) {
 // One radix pass: histogram digit `shift` of the values `digit_source(i)` over
 // the candidates with `participates(i)`, then locate the bin of rank `need`.
 template <bool FROM_TOP, typename Participates>
-__device__ inline void radix_pass(Shared& sh, uint32_t k0, uint32_t need, Participates digit_or_skip) {
+__device__ __forceinline__ void radix_pass(Shared& sh, uint32_t k0, uint32_t need, Participates digit_or_skip) {
   const uint32_t tid = threadIdx.x, nt = blockDim.x;
   uint32_t* my_copy = &sh.copies[(tid % kCopies) * kCopyStride];
   __syncthreads();
@@ -120,7 +120,7 @@ template <typename key_t> struct Cut {
 // key_at(i): order key of candidate i; index_at(i): its original index (only
 // read for candidates tied at T, and only when the tie group is cut).
 template <typename key_t, int KEY_BITS, typename KeyAt, typename IndexAt>
-__device__ inline Cut<key_t> find_cut(Shared& sh, uint32_t k0, uint32_t k, int index_bits, KeyAt key_at,
+__device__ __forceinline__ Cut<key_t> find_cut(Shared& sh, uint32_t k0, uint32_t k, int index_bits, KeyAt key_at,
                                       IndexAt index_at) {
   key_t prefix = 0, mask = 0;
   uint32_t need = k;
@@ -155,7 +155,7 @@ __device__ inline Cut<key_t> find_cut(Shared& sh, uint32_t k0, uint32_t k, int i
 // Stable compaction: wave w owns a contiguous run of candidates; emit(i, o)
 // is called for every surviving candidate i with its output slot o < k.
 template <typename Survives, typename Emit>
-__device__ inline void compact(Shared& sh, uint32_t k0, uint32_t k, Survives survives, Emit emit) {
+__device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Survives survives, Emit emit) {
   const uint32_t tid = threadIdx.x, nt = blockDim.x;
   const uint32_t waves = nt / kWave, wave = tid / kWave, lane = lane_id();
   uint32_t per_wave = (k0 + waves - 1) / waves;
