@@ -3,11 +3,12 @@
 // For batches of many moderate rows (a row's candidates fit in LDS) the
 // candidates never travel to HBM: the workgroup streams its row through the
 // same register queues as the streaming stage-1 kernel (stage1_stream.h),
-// parks the k0 candidates (raw value + sub-row number) in LDS, runs the
+// parks the k0 candidates (order key + sub-row number) in LDS, runs the
 // block-wide radix select of stage2_select.h over them and writes only the k
-// survivors.  HBM traffic is the input once plus the final k values and
-// indices per row; the two-kernel path additionally writes and re-reads
-// k0 * (sizeof(T) + 8) bytes per row.
+// survivors, whose values it gathers from the row (still in L2) so that they
+// are the input's bit patterns.  HBM traffic is the input once plus the final
+// k values and indices per row; the two-kernel path additionally writes and
+// re-reads k0 * (sizeof(T) + 8) bytes per row.
 //
 // Work split inside the workgroup: the row's T column tiles (64*V columns each)
 // are shared out over the waves; with few tiles, `split` waves share a tile,
@@ -31,21 +32,24 @@ using stream::kWave;
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
 __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
-    int64_t* __restrict__ indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t k0, uint32_t k,
-    int index_bits) {
+    int64_t* __restrict__ indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t hand_off,
+    uint32_t k0, uint32_t k, int index_bits) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
+  // keys are stored at their significant width
+  using skey_t = std::conditional_t<E::key_bits <= 16, uint16_t, key_t>;
   using Queue = stream::QueueFor<E, J, V, PACKED>;
   constexpr int kTileCols = kWave * V;
   constexpr int U = PACKED ? (V * J <= 8 ? 8 : 4) : (J <= 2 ? 8 : 4);
 
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   __shared__ select::Shared sh;
-  // candidates, then the hand-over area of the waves that share a tile
-  raw_t* cand_raw = reinterpret_cast<raw_t*>(dyn_lds);
-  const uint32_t pos_off = (k0 * (uint32_t)sizeof(raw_t) + 15u) & ~15u;
+  // Candidates, and the hand-over area of the waves that share a tile: behind
+  // the candidates, or (hand_off == 0, single round only) on top of them, in
+  // which case a barrier separates the last fold from the first candidate.
+  skey_t* cand_key = reinterpret_cast<skey_t*>(dyn_lds);
+  const uint32_t pos_off = (k0 * (uint32_t)sizeof(skey_t) + 15u) & ~15u;
   pos_t* cand_pos = reinterpret_cast<pos_t*>(dyn_lds + pos_off);
-  const uint32_t hand_off = (pos_off + k0 * (uint32_t)sizeof(pos_t) + 15u) & ~15u;
   const uint32_t nwaves = blockDim.x / kWave;
   unsigned char* hand = dyn_lds + hand_off;  // one Queue::kHandBytes area per wave that is not a tile leader
 
@@ -79,15 +83,15 @@ __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
         for (uint32_t w = 0; w + 1 < split; ++w)
           queue.fold_in(hand + (size_t)(group * (split - 1) + w) * Queue::kHandBytes, lane);
       }
+      if (hand_off == 0) __syncthreads();
     }
     if (live && part == 0) {
-      queue.fix_zeros(xr, g.b, col);
       ATK_STATIC_FOR(e, V * J) {
-        cand_raw[col * J + e] = queue.template raw<e / J, e % J>();
+        cand_key[col * J + e] = (skey_t)queue.template key<e / J, e % J>();
         cand_pos[col * J + e] = (pos_t)queue.template position<e / J, e % J>();
       } ATK_STATIC_END;
     }
-    if (split > 1) __syncthreads();  // the hand-over area is reused by the next round
+    if (split > 1 && hand_off != 0) __syncthreads();  // the hand-over area is reused by the next round
   }
 
   if (__syncthreads_or(any_nan)) {
@@ -105,12 +109,12 @@ __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
           stream::push_exact<E, J>(qv, qp, E::pad_raw, g.full_rows);
       }
 #pragma unroll
-      for (int s = 0; s < J; ++s) { cand_raw[c * J + s] = qv[s]; cand_pos[c * J + s] = (pos_t)qp[s]; }
+      for (int s = 0; s < J; ++s) { cand_key[c * J + s] = (skey_t)E::key(qv[s]); cand_pos[c * J + s] = (pos_t)qp[s]; }
     }
   }
   // (the select's first pass starts with a barrier, which also publishes the candidates)
 
-  auto key_at = [&](uint32_t i) -> key_t { return E::key(cand_raw[i]); };
+  auto key_at = [&](uint32_t i) -> key_t { return cand_key[i]; };
   auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)cand_pos[i] * (uint64_t)g.b + i / J; };
   const select::Cut<key_t> cut =
       select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
@@ -125,8 +129,9 @@ __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
         return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
       },
       [&](uint32_t i, uint32_t o) {
-        ov[o] = cand_raw[i];
-        oi[o] = (int64_t)index_at(i);
+        const int64_t index = (int64_t)index_at(i);
+        ov[o] = xr[index];
+        oi[o] = index;
       });
 }
 
@@ -143,6 +148,7 @@ struct Plan {
   bool pos16;           // sub-row numbers fit 16 bits
   bool packed;          // packed 16-bit queues
   int index_bits;
+  uint32_t hand_off;    // byte offset of the hand-over area in dynamic LDS (0: on top of the candidates)
   size_t lds_bytes;     // dynamic LDS
 };
 

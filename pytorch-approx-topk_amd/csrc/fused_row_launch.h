@@ -16,7 +16,7 @@ static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t row
       return ATK_ERR_LAUNCH;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(kWave * pl.waves), pl.lds_bytes, stream, x, values,
-                     indices, g, pl.tiles, pl.split, k0, k, pl.index_bits);
+                     indices, g, pl.tiles, pl.split, pl.hand_off, k0, k, pl.index_bits);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
@@ -34,9 +34,9 @@ template <typename E, int J>
 static int launch_j(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                     uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
   constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
-  if (pl.waves <= 4) {
-    return pl.pos16 ? launch_one<E, J, VF, 4, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
-                    : launch_one<E, J, VF, 4, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
+  if (pl.waves <= 8) {
+    return pl.pos16 ? launch_one<E, J, VF, 8, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
+                    : launch_one<E, J, VF, 8, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
   }
   return pl.pos16 ? launch_one<E, J, VF, 16, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
                   : launch_one<E, J, VF, 16, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);

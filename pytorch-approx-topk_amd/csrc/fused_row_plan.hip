@@ -8,17 +8,18 @@ namespace {
 // Rows below which one workgroup per row would leave most of the 256 CUs idle.
 constexpr int64_t kMinRows = 128;
 // Dynamic LDS a workgroup may use (candidates + hand-over); the select's own
-// block adds about 18 KiB.
+// block adds about 9 KiB.
 constexpr size_t kLdsBudget = 64 * 1024;
-// Waves per workgroup: 16, or 4 for the element types whose lanes own 8 columns
-// (their queues need the register budget of a small workgroup).
-inline uint32_t max_waves(int vec) { return vec <= 4 ? 16u : 4u; }
+// Waves per workgroup: 16, or 8 for the element types whose lanes own 8 columns
+// (their queues need the register budget of a smaller workgroup).
+inline uint32_t max_waves(int vec) { return vec <= 4 ? 16u : 8u; }
 }  // namespace
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned) {
   Plan pl{};
   pl.ok = false;
-  if (layout != ATK_INTERLEAVED && layout != ATK_INTERLEAVED_PADDED) return pl;
+  // (a padded row is never reduced further: its callers keep every bucket)
+  if (layout != ATK_INTERLEAVED) return pl;
   if (!aligned || rows < kMinRows || rows > 0x7fffffffll) return pl;
   if (k0 <= 0 || k <= 0 || k >= k0 || j < 1 || j > 4 || k0 % j) return pl;
   const int es = elem_bytes(dtype);
@@ -30,7 +31,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   if (b % pl.vec) return pl;
   pl.full_rows = (uint32_t)full;
   pl.rem = (uint32_t)(n - full * b);
-  pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
+  pl.pad_tail = 0;
   pl.pos16 = full + 1 <= 0xffff;
   pl.packed = (dtype == ATK_F16 || dtype == ATK_BF16 || dtype == ATK_I16) && full <= stream::kPackedMaxSubRow;
   const int64_t bound = (full + 1) * b;  // indices are < this
@@ -42,28 +43,39 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   // Worth it only when parking the candidates in HBM would cost a good part of
   // what reading the row costs: written and re-read k0*(es+8) bytes against n*es.
   if ((size_t)k0 * (es + 8) * 4 < (size_t)n * es) return pl;
-  const size_t cand_bytes = (((size_t)k0 * es + 15) & ~(size_t)15) +
+  const int skey = (dtype == ATK_U8 || dtype == ATK_I8) ? 2 : es;  // stored key width
+  const size_t cand_bytes = (((size_t)k0 * skey + 15) & ~(size_t)15) +
                             (((size_t)k0 * (pl.pos16 ? 2 : 4) + 15) & ~(size_t)15);
   if (cand_bytes > kLdsBudget) return pl;
 
   // Waves sharing a tile: as many as keep each share at least max(j, 8)
-  // sub-rows long, the workgroup within 16 waves and the hand-over within LDS.
+  // sub-rows long, the workgroup within its wave limit and LDS within budget.
+  // When all tiles are in flight at once the hand-over area may lie on top of
+  // the candidates.
   const int cmp_size = es > 4 ? 8 : 4;
   const int64_t min_run = j > 8 ? j : 8;
   const uint32_t kMaxWaves = max_waves(pl.vec);
+  auto hand_bytes = [&](uint32_t split) {
+    const uint32_t waves = pl.tiles * split <= kMaxWaves ? pl.tiles * split : kMaxWaves;
+    return (size_t)(waves - waves / split) * pl.vec * j * stream::kWave * (cmp_size + 4);
+  };
+  auto lds_need = [&](uint32_t split) {
+    const bool one_round = pl.tiles * split <= kMaxWaves;
+    const size_t hand = hand_bytes(split);
+    return one_round ? (hand > cand_bytes ? hand : cand_bytes) : cand_bytes + hand;
+  };
   uint32_t split = 1;
   if (pl.tiles < kMaxWaves) {
     for (uint32_t cand = 2; cand * pl.tiles <= kMaxWaves; cand *= 2) {
-      if (full / cand < min_run) break;
-      const size_t hand = (size_t)pl.tiles * (cand - 1) * pl.vec * j * stream::kWave * (cmp_size + 4);
-      if (cand_bytes + hand > kLdsBudget) break;
+      if (full / cand < min_run || lds_need(cand) > kLdsBudget) break;
       split = cand;
     }
   }
   pl.split = split;
   pl.waves = pl.tiles * split <= kMaxWaves ? pl.tiles * split : kMaxWaves;
-  const uint32_t helpers = pl.waves - pl.waves / split;
-  pl.lds_bytes = cand_bytes + (size_t)helpers * pl.vec * j * stream::kWave * (cmp_size + 4);
+  const bool one_round = pl.tiles * split <= kMaxWaves;
+  pl.hand_off = (split > 1 && !one_round) ? (uint32_t)cand_bytes : 0u;
+  pl.lds_bytes = lds_need(split);
   pl.ok = true;
   return pl;
 }

@@ -234,6 +234,8 @@ template <typename E, int J, int V> struct CmpQueue {
     } ATK_STATIC_END;
   }
   __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t) {}
+  // exact order key of an entry (the queues are not poisoned)
+  template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return E::key(C::to_raw(q[VI][SI])); }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const { return C::to_raw(q[VI][SI]); }
   template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return pos[VI][SI]; }
 };
@@ -365,6 +367,8 @@ template <typename E, int J, int V> struct PackedQueue {
       } ATK_STATIC_END;
     }
   }
+  // exact order key of an entry: without NaN the packed key is the exact key
+  template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return q[VI][SI] >> 16; }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
     const raw_t r = K::unkey(q[VI][SI] >> 16);
     if constexpr (K::zero_is_ambiguous) return (neg_zeros >> (VI * J + SI)) & 1u ? (raw_t)0x8000u : r;

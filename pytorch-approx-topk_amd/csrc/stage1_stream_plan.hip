@@ -1,6 +1,4 @@
 // Host-side planning and dispatch of the streaming stage-1 kernels.
-#include <cstdlib>
-
 #include "stage1_stream.h"
 
 namespace atk {
@@ -37,18 +35,23 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   pl.col_tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
 
   // Waves per workgroup.  Wave 0's serial work per column is its own run,
-  // full/w pushes, plus (w-1)*j pushes to fold the other waves' queues; take
-  // the w that minimises it (the larger on a tie: short-lived waves keep more
-  // of the HBM bandwidth), with every run at least j long and the LDS
-  // hand-over within its budget.
+  // full/w pushes, plus (w-1)*j pushes to fold the other waves' queues.  Take
+  // the largest w within 30 % of the cheapest (short-lived waves keep more of
+  // the HBM bandwidth: measured, 8 waves x 4 sub-rows beats 4 x 8 at the
+  // headline shape), with every run at least j long and the LDS hand-over
+  // within its budget.
   const int cmp_size = es > 4 ? 8 : 4;
-  int w = 1;
-  int64_t best = full;
-  for (int cand = 2; cand <= 8; cand *= 2) {
+  int64_t cost[4] = {full, 0, 0, 0};
+  int cands = 1;
+  for (int cand = 2; cand <= 8; cand *= 2, ++cands) {
     if (full / cand < j || merge_lds_bytes(pl.vec, j, cand, cmp_size) > kMergeLdsLimit) break;
-    const int64_t cost = full / cand + (int64_t)(cand - 1) * j;
-    if (cost <= best) { best = cost; w = cand; }
+    cost[cands] = full / cand + (int64_t)(cand - 1) * j;
   }
+  int64_t best = cost[0];
+  for (int i = 1; i < cands; ++i) best = cost[i] < best ? cost[i] : best;
+  int w = 1;
+  for (int i = 0; i < cands; ++i)
+    if (cost[i] * 10 <= best * 13) w = 1 << i;
   pl.waves = w;
 
   // Slabs: only when the grid would still be small and the runs are long.
@@ -60,13 +63,6 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
     if (slabs > most) slabs = most;
     if (slabs < 1) slabs = 1;
     pl.slabs = (uint32_t)slabs;
-  }
-  if (const char* e = getenv("ATK_TUNE_WAVES")) {
-    const int tw = atoi(e);
-    if ((tw == 1 || tw == 2 || tw == 4 || tw == 8) && full / tw >= j &&
-        merge_lds_bytes(pl.vec, j, tw, cmp_size) <= kMergeLdsLimit)
-      pl.waves = tw;
-    if (const char* s = getenv("ATK_TUNE_SLABS")) pl.slabs = (uint32_t)atoi(s);
   }
   pl.slab_len = (uint32_t)(full / pl.slabs);
   // every wave scans exactly 4 or 8 sub-rows: straight-line kernels exist for that

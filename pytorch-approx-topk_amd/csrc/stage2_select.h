@@ -24,7 +24,7 @@ constexpr int kMaxWaves = 16;
 // one) so that the many candidates sharing a digit -- the top byte of a float
 // key is nearly constant among top-k candidates -- do not serialise on one LDS
 // address; the odd stride spreads equal digits of different copies over banks.
-constexpr int kCopies = 16;
+constexpr int kCopies = 8;
 constexpr int kCopyStride = 257;
 
 struct Shared {
@@ -100,8 +100,18 @@ __device__ __forceinline__ void radix_pass(Shared& sh, uint32_t k0, uint32_t nee
   __syncthreads();
   for (uint32_t i = tid; i < kCopies * kCopyStride; i += nt) sh.copies[i] = 0;
   __syncthreads();
-  for (uint32_t i = tid; i < k0; i += nt) {
-    const int d = digit_or_skip(i);  // 0..255, or -1 when candidate i is out of the race
+  // four candidates per trip, so that their LDS reads and adds overlap
+  uint32_t i = tid;
+  for (; i + 3 * nt < k0; i += 4 * nt) {
+    int d[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) d[u] = digit_or_skip(i + u * nt);  // 0..255, or -1: out of the race
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (d[u] >= 0) atomicAdd(&my_copy[d[u]], 1u);
+  }
+  for (; i < k0; i += nt) {
+    const int d = digit_or_skip(i);
     if (d >= 0) atomicAdd(&my_copy[d], 1u);
   }
   __syncthreads();
@@ -162,7 +172,15 @@ __device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Sur
   per_wave = (per_wave + kWave - 1) / kWave * kWave;
   const uint32_t lo = min(wave * per_wave, k0), hi = min(lo + per_wave, k0);
   uint32_t mine = 0;
-  for (uint32_t base = lo; base < hi; base += kWave) {
+  uint32_t base = lo;
+  for (; base + 4 * kWave <= hi; base += 4 * kWave) {  // four groups per trip: independent LDS reads
+    bool sel[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) sel[u] = survives(base + u * kWave + lane);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) mine += (uint32_t)__popcll(__ballot(sel[u]));
+  }
+  for (; base < hi; base += kWave) {
     const uint32_t i = base + lane;
     const bool sel = i < hi && survives(i);
     mine += (uint32_t)__popcll(__ballot(sel));
@@ -172,7 +190,22 @@ __device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Sur
   __syncthreads();
   uint32_t out = 0;
   for (uint32_t w = 0; w < wave; ++w) out += sh.wave_total[w];
-  for (uint32_t base = lo; base < hi; base += kWave) {
+  base = lo;
+  for (; base + 4 * kWave <= hi; base += 4 * kWave) {
+    bool sel[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) sel[u] = survives(base + u * kWave + lane);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint64_t m = __ballot(sel[u]);
+      if (sel[u]) {
+        const uint32_t o = out + rank_in(m);
+        if (o < k) emit(base + u * kWave + lane, o);
+      }
+      out += (uint32_t)__popcll(m);
+    }
+  }
+  for (; base < hi; base += kWave) {
     const uint32_t i = base + lane;
     const bool sel = i < hi && survives(i);
     const uint64_t m = __ballot(sel);
