@@ -128,8 +128,8 @@ __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
         if (key != cut.T) return key > cut.T;
         return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
       },
-      [&](uint32_t i, uint32_t o) {
-        const int64_t index = (int64_t)index_at(i);
+      [&](uint32_t i) { return (int64_t)index_at(i); },
+      [&](uint32_t, uint32_t o, int64_t index) {
         ov[o] = xr[index];
         oi[o] = index;
       });

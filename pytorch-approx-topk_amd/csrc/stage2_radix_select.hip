@@ -12,6 +12,8 @@ namespace atk {
 
 namespace {
 
+template <typename raw_t> struct Candidate { raw_t value; int64_t index; };
+
 template <typename E, bool KEYS_IN_LDS>
 __global__ __launch_bounds__(1024) void select_kernel(
     const typename E::raw_t* __restrict__ cand_values,
@@ -28,7 +30,16 @@ __global__ __launch_bounds__(1024) void select_kernel(
   const int64_t* ci = cand_indices + row * (int64_t)k0;
 
   if (KEYS_IN_LDS) {
-    for (uint32_t i = threadIdx.x; i < k0; i += blockDim.x) keys[i] = E::key(cv[i]);
+    // eight loads in flight per lane
+    uint32_t i = threadIdx.x;
+    for (; i + 7 * blockDim.x < k0; i += 8 * blockDim.x) {
+      raw_t got[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) got[u] = cv[i + u * blockDim.x];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) keys[i + u * blockDim.x] = E::key(got[u]);
+    }
+    for (; i < k0; i += blockDim.x) keys[i] = E::key(cv[i]);
   }
   auto key_at = [&](uint32_t i) -> key_t { return KEYS_IN_LDS ? keys[i] : E::key(cv[i]); };
   auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)ci[i]; };
@@ -45,7 +56,8 @@ __global__ __launch_bounds__(1024) void select_kernel(
         if (key != cut.T) return key > cut.T;
         return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
       },
-      [&](uint32_t i, uint32_t o) { ov[o] = cv[i]; oi[o] = ci[i]; });
+      [&](uint32_t i) { return Candidate<raw_t>{cv[i], ci[i]}; },
+      [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) { ov[o] = c.value; oi[o] = c.index; });
 }
 
 // LDS a workgroup may use for keys; the rest of the 160 KB of a gfx950 CU is

@@ -162,10 +162,14 @@ __device__ __forceinline__ Cut<key_t> find_cut(Shared& sh, uint32_t k0, uint32_t
   return cut;
 }
 
-// Stable compaction: wave w owns a contiguous run of candidates; emit(i, o)
-// is called for every surviving candidate i with its output slot o < k.
-template <typename Survives, typename Emit>
-__device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Survives survives, Emit emit) {
+// Stable compaction: wave w owns a contiguous run of candidates.  fetch(i) is
+// called for every candidate of a group before any of them is tested, so that
+// its loads (coalesced, independent of the outcome) overlap; emit(i, o, what
+// fetch(i) returned) is called for every surviving candidate i with its output
+// slot o < k.
+template <typename Survives, typename Fetch, typename Emit>
+__device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Survives survives, Fetch fetch,
+                                        Emit emit) {
   const uint32_t tid = threadIdx.x, nt = blockDim.x;
   const uint32_t waves = nt / kWave, wave = tid / kWave, lane = lane_id();
   uint32_t per_wave = (k0 + waves - 1) / waves;
@@ -190,9 +194,13 @@ __device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Sur
   __syncthreads();
   uint32_t out = 0;
   for (uint32_t w = 0; w < wave; ++w) out += sh.wave_total[w];
+  using Fetched = decltype(fetch(0u));
   base = lo;
   for (; base + 4 * kWave <= hi; base += 4 * kWave) {
+    Fetched got[4];
     bool sel[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) got[u] = fetch(base + u * kWave + lane);
 #pragma unroll
     for (int u = 0; u < 4; ++u) sel[u] = survives(base + u * kWave + lane);
 #pragma unroll
@@ -200,7 +208,7 @@ __device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Sur
       const uint64_t m = __ballot(sel[u]);
       if (sel[u]) {
         const uint32_t o = out + rank_in(m);
-        if (o < k) emit(base + u * kWave + lane, o);
+        if (o < k) emit(base + u * kWave + lane, o, got[u]);
       }
       out += (uint32_t)__popcll(m);
     }
@@ -211,7 +219,7 @@ __device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Sur
     const uint64_t m = __ballot(sel);
     if (sel) {
       const uint32_t o = out + rank_in(m);
-      if (o < k) emit(i, o);
+      if (o < k) emit(i, o, fetch(i));
     }
     out += (uint32_t)__popcll(m);
   }
