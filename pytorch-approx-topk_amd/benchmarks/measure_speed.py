@@ -1,0 +1,100 @@
+#!/usr/bin/env python3
+"""Runtime sweep of exact and approximate top-k on one GPU, written as JSON lines.
+
+Covers the grid of the reference's benchmarks/measure_speed.py:264-327
+(n in 2^12..2^16, batch in {128, 32}, k in {64, n/8}, fp32; torch.topk, the
+approximate top-k at j in {1, 2, 4}, and the torch-level bucketed arg-max), once
+with plain launches and once with the inner loop captured in a HIP graph, timed
+with events as benchmarks/measure_speed.py:98-146 does.  Every line carries the
+per-call durations in seconds; input bandwidth is dtype_bytes * n * batch / mean
+(benchmarks/plot_bandwidth.py:41-45).
+
+    python pytorch-approx-topk_amd/benchmarks/measure_speed.py [--out results.jsonl] [--quick]
+"""
+from __future__ import annotations
+
+import argparse
+import itertools
+import json
+import os
+import sys
+from typing import Any, Callable
+
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+from approx_topk import topk as approx_topk  # noqa: E402
+from approx_topk.experimental import bucketed_argmax  # noqa: E402
+
+
+def exact_topk(xs, k, dim):
+    return torch.topk(xs, k, dim, sorted=False)
+
+
+def time_calls(call: Callable[[int], Any], refresh: Callable[[], None], n_outer: int, n_inner: int,
+               graph: bool, n_warmup: int = 16) -> list[float]:
+    """Seconds per call for `n_outer` timed repetitions of `n_inner` calls each."""
+    def inner():
+        return [call(i) for i in range(n_inner)]
+
+    run = inner
+    if graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            refresh()
+            inner()
+        torch.cuda.current_stream().wait_stream(side)
+        captured = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(captured):
+            keep = inner()  # noqa: F841  (outputs stay alive with the graph)
+        run = captured.replay
+    for _ in range(n_warmup):
+        refresh()
+        run()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range(n_outer)]
+    for start, stop in events:
+        refresh()
+        start.record()
+        run()
+        stop.record()
+    torch.cuda.synchronize()
+    return [start.elapsed_time(stop) / 1e3 / n_inner for start, stop in events]
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--out", default="measure_speed.jsonl")
+    ap.add_argument("--quick", action="store_true", help="fewer repetitions")
+    args = ap.parse_args()
+
+    methods: list[tuple[str, Callable, dict]] = [("torch.topk", exact_topk, {})]
+    for j in (1, 2, 4):
+        methods.append((f"approx_topk.topk j={j}", approx_topk, dict(j=j, k_mult=1)))
+    methods.append(("bucketed_argmax.topk_torch", bucketed_argmax.topk_torch, dict(interleaved=True)))
+
+    modes = [dict(graph=False, n_outer=64 if args.quick else 512, n_inner=1),
+             dict(graph=True, n_outer=4 if args.quick else 16, n_inner=128)]
+    device = torch.cuda.get_device_name()
+    with open(args.out, "w") as out:
+        for exp, batch, mode in itertools.product([16, 15, 14, 13, 12], [128, 32], modes):
+            n = 2 ** exp
+            xs = torch.zeros(mode["n_inner"], batch, n, device="cuda")
+            for k in (64, n // 8):
+                for name, fn, kwargs in methods:
+                    durations = time_calls(lambda i: fn(xs[i], k=k, dim=1, **kwargs)[0],
+                                           lambda: xs.normal_(), **mode)
+                    mean = sum(durations) / len(durations)
+                    row = dict(method=name, args=kwargs, batch_size=batch, topk_size=n, k=k, dtype="float32",
+                               hip_graphs=mode["graph"], n_outer=mode["n_outer"], n_inner=mode["n_inner"],
+                               duration=durations, input_GBps=4 * n * batch / mean / 1e9, device=device)
+                    print(json.dumps(row), file=out, flush=True)
+                    print(f"n=2^{exp} batch={batch} k={k} graph={mode['graph']} {name}: "
+                          f"{mean * 1e6:.1f} us, {row['input_GBps']:.0f} GB/s", flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -49,7 +49,7 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
   Geom g{};
   g.row_stride = row_stride; g.b = k0 / j;
   g.full_rows = pl.full_rows; g.rem = pl.rem; g.pad_tail = pl.pad_tail;
-  g.slabs = 1; g.slab_len = pl.full_rows; g.col_tiles = pl.tiles;
+  g.slabs = 1; g.slab_len = pl.full_rows; g.col_tiles = pl.tiles; g.fold = 1;
   const raw_t* xs = static_cast<const raw_t*>(x);
   raw_t* ov = static_cast<raw_t*>(values);
   switch (j) {

@@ -380,20 +380,27 @@ template <typename E, int J, int V> struct PackedQueue {
 template <typename E, int J, int V, bool PACKED>
 using QueueFor = std::conditional_t<PACKED, PackedQueue<E, J, V>, CmpQueue<E, J, V>>;
 
-// Shape of one launch; passed to the kernels by value.
+// Shape of one launch; passed to the kernels by value.  With few buckets the
+// planner folds the row: `fold` consecutive sub-rows of the true [L][b] matrix
+// form one sub-row of a matrix with b * fold columns, which is what the kernel
+// scans; column f*b + c of it holds every fold-th element of bucket c, the flat
+// index of an element is the same in both views, and the merge kernel folds the
+// `fold` columns of a bucket back together.  `b` below is the scanned width.
 struct Geom {
   int64_t row_stride;     // elements between rows
-  int64_t b;              // buckets (columns) per row
+  int64_t b;              // columns per row as scanned
   uint32_t full_rows;     // L = n / b
   uint32_t rem;           // n mod b: columns that have one more element
   uint32_t pad_tail;      // padded row: the other columns hold the pad value there
   uint32_t slabs;         // sub-row slabs per row
   uint32_t slab_len;      // sub-rows per slab (the last slab takes the rest)
   uint32_t col_tiles;     // workgroup column tiles per row
+  uint32_t fold;          // > 1: the kernel itself merges the folded columns (one workgroup per row)
 };
 
-// Where results go: final values/indices[rows][b*J] when there is one slab,
-// else per-slab queues [rows][slabs][b*J] (raw values and sub-row numbers).
+// Where results go: final values/indices[rows][b*J], or, when the merge kernel
+// follows (several slabs, or a folded row; part_values != nullptr), per-slab
+// queues [rows][slabs][b*J] (raw values and sub-row numbers).
 template <typename raw_t> struct Sink {
   raw_t* values;
   int64_t* indices;
@@ -407,7 +414,7 @@ template <typename E, int J, int V, typename Queue>
 __device__ __forceinline__ void emit(const Geom& g, const Sink<typename E::raw_t>& out, int64_t row,
                                      uint32_t slab, int64_t col, const Queue& queue) {
   using raw_t = typename E::raw_t;
-  if (g.slabs == 1) {
+  if (out.part_values == nullptr) {
     const int64_t o = (row * g.b + col) * J;
     raw_t* ov = out.values + o;
     int64_t* oi = out.indices + o;
@@ -470,7 +477,7 @@ __device__ __forceinline__ void exact_columns(const typename E::raw_t* __restric
       else if (g.pad_tail)
         push_exact<E, J>(val, pos, E::pad_raw, g.full_rows);
     }
-    if (g.slabs == 1) {
+    if (out.part_values == nullptr) {
       const int64_t o = (row * g.b + c) * J;
 #pragma unroll
       for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices[o + s] = c + (int64_t)pos[s] * g.b; }
@@ -562,6 +569,135 @@ __device__ __forceinline__ void scan_run(const typename E::raw_t* __restrict__ x
   }
 }
 
+// An entry while partial queues are merged: order key and sub-row number in one comparable
+// word (a larger word is a better entry; the all-zero word is an empty slot,
+// which no entry equals because sub-row numbers stay below 0xfffffffe).
+template <typename E, bool WIDE = (E::key_bits > 32)> struct MergeWord {
+  using word_t = uint64_t;
+  __device__ static __forceinline__ word_t make(typename E::raw_t raw, uint32_t p) {
+    return ((uint64_t)E::key(raw) << 32) | (uint64_t)(0xffffffffu - p);
+  }
+  __device__ static __forceinline__ word_t empty() { return 0; }
+  __device__ static __forceinline__ bool better(word_t a, word_t b) { return a > b; }
+  __device__ static __forceinline__ uint32_t pos(word_t w) { return 0xffffffffu - (uint32_t)w; }
+  __device__ static __forceinline__ word_t from_lane(word_t w, int lane) { return __shfl(w, lane); }
+};
+template <typename E> struct MergeWord<E, true> {
+  struct word_t { uint64_t key; uint32_t npos; uint32_t unused; };
+  __device__ static __forceinline__ word_t make(typename E::raw_t raw, uint32_t p) {
+    return word_t{E::key(raw), 0xffffffffu - p, 0u};
+  }
+  __device__ static __forceinline__ word_t empty() { return word_t{0, 0, 0}; }
+  __device__ static __forceinline__ bool better(const word_t& a, const word_t& b) {
+    return a.key > b.key || (a.key == b.key && a.npos > b.npos);
+  }
+  __device__ static __forceinline__ uint32_t pos(const word_t& w) { return 0xffffffffu - w.npos; }
+  __device__ static __forceinline__ word_t from_lane(const word_t& w, int lane) {
+    return word_t{__shfl(w.key, lane), __shfl(w.npos, lane), 0u};
+  }
+};
+
+// acc and in are ascending lists of N entries (N a power of two); acc becomes
+// the N best of both, ascending: the element-wise better of acc and reversed
+// `in` is a bitonic sequence holding exactly those, which half-cleaners sort.
+template <typename M, int N>
+__device__ __forceinline__ void merge_best(typename M::word_t (&acc)[N], const typename M::word_t (&in)[N]) {
+  ATK_STATIC_FOR(i, N) { if (M::better(in[N - 1 - i], acc[i])) acc[i] = in[N - 1 - i]; } ATK_STATIC_END;
+  auto order = [&](auto lo, auto hi) __attribute__((always_inline)) {
+    const bool swap = M::better(acc[lo], acc[hi]);
+    const typename M::word_t a = acc[lo], b = acc[hi];
+    acc[lo] = swap ? b : a;
+    acc[hi] = swap ? a : b;
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  static_assert(N == 1 || N == 2 || N == 4, "queues hold at most four entries");
+  if constexpr (N == 4) { order(I0{}, I2{}); order(I1{}, I3{}); order(I0{}, I1{}); order(I2{}, I3{}); }
+  if constexpr (N == 2) { order(I0{}, I1{}); }
+}
+
+// The last step of a folded row that one workgroup scanned alone (wave 0, all
+// 64 lanes, after the waves' queues are folded): the `fold` scanned columns of
+// every bucket are merged and the final result written.  The queues go to LDS
+// as merge words; cb lanes (a power of two) then cover cb buckets at a time
+// with 64/cb lanes per bucket, which share out the bucket's columns and
+// combine pairwise by lane shuffles.
+template <typename E, int J, int V, typename Queue>
+__device__ __forceinline__ void fold_columns(const typename E::raw_t* __restrict__ xr, const Geom& g,
+                                             const Sink<typename E::raw_t>& out, int64_t row, int64_t col,
+                                             bool live, uint32_t lane, const Queue& queue,
+                                             unsigned char* lds) {
+  using M = MergeWord<E>;
+  using word_t = typename M::word_t;
+  constexpr int N = J == 3 ? 4 : J;
+  word_t* words = reinterpret_cast<word_t*>(lds);  // [scanned column][J]
+  const uint32_t b = (uint32_t)g.b / g.fold;       // buckets
+  if (live) {
+    ATK_STATIC_FOR(v, V) {
+      const uint32_t cw = (uint32_t)col + v;
+      const uint32_t f = cw / b;
+      ATK_STATIC_FOR(sl, J) {
+        words[cw * J + sl] = M::make(queue.template raw<v, sl>(), queue.template position<v, sl>() * g.fold + f);
+      } ATK_STATIC_END;
+    } ATK_STATIC_END;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  uint32_t cb = kWave;
+  while (cb > 1 && cb / 2 >= b) cb /= 2;
+  const uint32_t share = lane / cb, shares = kWave / cb;
+  for (uint32_t c0 = 0; c0 < b; c0 += cb) {  // the same trips for every lane
+    const uint32_t c = c0 + lane % cb;
+    word_t acc[N], in[N];
+    ATK_STATIC_FOR(sl, N) { acc[sl] = M::empty(); in[sl] = M::empty(); } ATK_STATIC_END;
+    if (c < b) {
+      for (uint32_t f = share; f < g.fold; f += shares) {
+        ATK_STATIC_FOR(sl, J) { in[N - J + sl] = words[(f * b + c) * J + sl]; } ATK_STATIC_END;
+        merge_best<M, N>(acc, in);
+      }
+    }
+    for (uint32_t half = shares / 2; half >= 1; half /= 2) {
+      ATK_STATIC_FOR(sl, N) { in[sl] = M::from_lane(acc[sl], (int)(lane + half * cb)); } ATK_STATIC_END;
+      merge_best<M, N>(acc, in);  // meaningful in the lanes with share < half, which are the ones read next
+    }
+    if (share == 0 && c < b) {
+      const int64_t o = (row * b + c) * J;
+      ATK_STATIC_FOR(sl, J) {
+        const int64_t index = c + (int64_t)M::pos(acc[N - J + sl]) * b;
+        out.values[o + sl] = xr[index];
+        out.indices[o + sl] = index;
+      } ATK_STATIC_END;
+    }
+  }
+}
+
+// The same result through order keys, one lane per bucket walking the whole
+// bucket: taken when the row holds a value the fast queues cannot order.
+template <typename E, int J>
+__device__ __forceinline__ void fold_columns_exact(const typename E::raw_t* __restrict__ xr, const Geom& g,
+                                                   const Sink<typename E::raw_t>& out, int64_t row,
+                                                   uint32_t lane) {
+  using raw_t = typename E::raw_t;
+  const uint32_t b = (uint32_t)g.b / g.fold;
+  const uint32_t length = g.full_rows * g.fold + g.rem / b, rem = g.rem % b;
+  for (uint32_t c = lane; c < b; c += kWave) {
+    raw_t val[J];
+    uint32_t pos[J];
+    clear_exact<E, J>(val, pos);
+    for (uint32_t p = 0; p < length; ++p) push_exact<E, J>(val, pos, xr[(int64_t)p * b + c], p);
+    if (rem != 0) {
+      if (c < rem) push_exact<E, J>(val, pos, xr[(int64_t)length * b + c], length);
+      else if (g.pad_tail) push_exact<E, J>(val, pos, E::pad_raw, length);
+    }
+    const int64_t o = (row * b + c) * J;
+#pragma unroll
+    for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices[o + s] = c + (int64_t)pos[s] * b; }
+  }
+}
+
 // E: element traits; J: entries kept per bucket; V: columns per lane; W: waves
 // per workgroup, sharing one column tile and splitting its sub-rows; U: loads
 // kept in flight per lane; RUN: exact sub-rows per wave when known (else 0);
@@ -598,16 +734,29 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
   scan_run<E, J, V, U, RUN>(xr, g, col, live, p0, p1, last_slab && wave == W - 1, queue);
 
   bool redo = queue.poisoned();
+  // LDS: the hand-over area of waves 1.., later the merge words of a folded row
+  using word_t = typename MergeWord<E>::word_t;
+  constexpr size_t kHandArea = (size_t)(W - 1) * Queue::kHandBytes;
+  constexpr size_t kWordArea = (size_t)kTileCols * J * sizeof(word_t);
+  __shared__ __align__(16) unsigned char lds[kHandArea > kWordArea ? kHandArea : kWordArea];
   if constexpr (W > 1) {
     // waves 1.. hand their queues to wave 0 through LDS
-    __shared__ __align__(16) unsigned char hand[(W - 1) * Queue::kHandBytes];
-    if (wave > 0) queue.hand_over(hand + (size_t)(wave - 1) * Queue::kHandBytes, lane);
+    if (wave > 0) queue.hand_over(lds + (size_t)(wave - 1) * Queue::kHandBytes, lane);
     redo = __syncthreads_or(redo);
     if (wave > 0) return;
     if (!redo) {
 #pragma nounroll
-      for (int w = 0; w < W - 1; ++w) queue.fold_in(hand + (size_t)w * Queue::kHandBytes, lane);
+      for (int w = 0; w < W - 1; ++w) queue.fold_in(lds + (size_t)w * Queue::kHandBytes, lane);
     }
+  }
+  if (g.fold > 1) {
+    if (redo) {
+      fold_columns_exact<E, J>(xr, g, out, row, lane);
+    } else {
+      if (live) queue.fix_zeros(xr, g.b, col);
+      fold_columns<E, J, V>(xr, g, out, row, col, live, lane, queue, lds);
+    }
+    return;
   }
   if (!live) return;
   if (redo) {
@@ -618,53 +767,65 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
   emit<E, J, V>(g, out, row, slab, col, queue);
 }
 
-// Folds the per-slab queues of every bucket into the final result with exact
-// order keys.  A workgroup of 4 waves covers 64 buckets (one per lane); wave w
-// folds a contiguous quarter of the slabs, then waves 1..3 hand their queues to
-// wave 0 through LDS.  Slabs are visited in sub-row order and each queue's
-// entries best first, so equal values keep the lowest index.
-constexpr int kMergeWaves = 4;
+// Folds the partial queues of every bucket into the final result under the
+// full order (order key, then lower index).  A bucket has slabs * fold partial
+// queues ("sources"): source (slab, f) is column f*b + c of that slab's scanned
+// matrix, and its entry at scanned sub-row q is the bucket's element number
+// q*fold + f.  A workgroup of 256 threads covers `cb` buckets (a power of two
+// up to 64) with 256/cb threads per bucket, which share the sources out and
+// then combine pairwise through LDS.  Every partial queue arrives ascending,
+// so combining two is a merge network, not J insertions.  The winners' values
+// are read back from the row, so that they are the input's bit patterns.
+constexpr int kMergeThreads = 256;
 
 template <typename E, int J>
-__global__ __launch_bounds__(kWave * kMergeWaves) void stream_merge_kernel(
+__global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
+    const typename E::raw_t* __restrict__ x, int64_t row_stride,
     const typename E::raw_t* __restrict__ part_values, const uint32_t* __restrict__ part_pos,
-    int64_t b, uint32_t slabs, int64_t blocks_per_row, typename E::raw_t* __restrict__ values,
-    int64_t* __restrict__ indices) {
-  using raw_t = typename E::raw_t;
-  __shared__ raw_t lds_q[kMergeWaves - 1][J][kWave];
-  __shared__ uint32_t lds_p[kMergeWaves - 1][J][kWave];
-  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int64_t row = blockIdx.x / blocks_per_row;
-  const int64_t c = (blockIdx.x - row * blocks_per_row) * kWave + lane;
+    int64_t b, uint32_t fold, uint32_t slabs, uint32_t cb, uint32_t blocks_per_row,
+    typename E::raw_t* __restrict__ values, int64_t* __restrict__ indices) {
+  using M = MergeWord<E>;
+  using word_t = typename M::word_t;
+  constexpr int N = J == 3 ? 4 : J;  // list length of the merge network
+  __shared__ word_t lds[N][kMergeThreads];
+  const uint32_t t = threadIdx.x;
+  const uint32_t share = t / cb, shares = kMergeThreads / cb;
+  const uint32_t row32 = blockIdx.x / blocks_per_row;
+  const int64_t row = row32;
+  const int64_t c = (int64_t)(blockIdx.x - row32 * blocks_per_row) * cb + t % cb;
   const bool live = c < b;
-  raw_t q[J];
-  uint32_t pos[J];
-  clear_exact<E, J>(q, pos);
-  const uint32_t lo = (uint32_t)(((uint64_t)slabs * wave) / kMergeWaves);
-  const uint32_t hi = (uint32_t)(((uint64_t)slabs * (wave + 1)) / kMergeWaves);
+  const int64_t width = b * fold;
+  word_t acc[N], in[N];
+  ATK_STATIC_FOR(s, N) { acc[s] = M::empty(); in[s] = M::empty(); } ATK_STATIC_END;
   if (live) {
-    for (uint32_t slab = lo; slab < hi; ++slab) {
-      const int64_t o = ((row * slabs + slab) * b + c) * J;
-#pragma unroll
-      for (int s = J - 1; s >= 0; --s) push_exact<E, J>(q, pos, part_values[o + s], part_pos[o + s]);
+    const uint32_t sources = slabs * fold;
+    uint32_t slab = share / fold, f = share - slab * fold;
+    for (uint32_t src = share; src < sources; src += shares) {
+      const int64_t o = ((row * slabs + slab) * width + (int64_t)f * b + c) * J;
+      ATK_STATIC_FOR(s, J) { in[N - J + s] = M::make(part_values[o + s], part_pos[o + s] * fold + f); } ATK_STATIC_END;
+      merge_best<M, N>(acc, in);
+      f += shares;
+      while (f >= fold) { f -= fold; ++slab; }
     }
   }
-  if (wave > 0) {
-#pragma unroll
-    for (int s = 0; s < J; ++s) { lds_q[wave - 1][s][lane] = q[s]; lds_p[wave - 1][s][lane] = pos[s]; }
+  for (uint32_t half = shares / 2; half >= 1; half /= 2) {
+    if (share >= half && share < 2 * half) {
+      ATK_STATIC_FOR(s, N) { lds[s][t] = acc[s]; } ATK_STATIC_END;
+    }
+    __syncthreads();
+    if (share < half) {
+      ATK_STATIC_FOR(s, N) { in[s] = lds[s][t + half * cb]; } ATK_STATIC_END;
+      merge_best<M, N>(acc, in);
+    }
   }
-  __syncthreads();
-  if (wave > 0 || !live) return;
-  for (int w = 1; w < kMergeWaves; ++w) {
-    const uint32_t wlo = (uint32_t)(((uint64_t)slabs * w) / kMergeWaves);
-    const uint32_t whi = (uint32_t)(((uint64_t)slabs * (w + 1)) / kMergeWaves);
-    if (whi == wlo) continue;  // that wave had no slab
-#pragma unroll
-    for (int s = J - 1; s >= 0; --s) push_exact<E, J>(q, pos, lds_q[w - 1][s][lane], lds_p[w - 1][s][lane]);
-  }
+  if (share != 0 || !live) return;
+  const typename E::raw_t* xr = x + row * row_stride;
   const int64_t o = (row * b + c) * J;
-#pragma unroll
-  for (int s = 0; s < J; ++s) { values[o + s] = q[s]; indices[o + s] = c + (int64_t)pos[s] * b; }
+  ATK_STATIC_FOR(s, J) {
+    const int64_t index = c + (int64_t)M::pos(acc[N - J + s]) * b;
+    values[o + s] = xr[index];
+    indices[o + s] = index;
+  } ATK_STATIC_END;
 }
 
 // ---------------------------------------------------------------------------
@@ -677,8 +838,11 @@ struct Plan {
   int waves;          // W: waves per workgroup (1, 2, 4 or 8)
   bool packed;        // packed 16-bit queues (16-bit element type, short enough rows)
   int run;            // sub-rows per wave when every wave gets exactly 4 or 8, else 0
-  uint32_t full_rows, rem, pad_tail;
+  uint32_t fold;      // sub-rows of the true matrix per scanned sub-row (1: not folded)
+  int64_t width;      // scanned columns per row: buckets * fold
+  uint32_t full_rows, rem, pad_tail;  // of the scanned matrix
   uint32_t slabs, slab_len, col_tiles;
+  bool merge;         // the merge kernel follows (several slabs or a folded row)
   size_t part_values_off, part_pos_off, ws_bytes;
 };
 
@@ -687,8 +851,8 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
 
 // One instance per element type, each in its own translation unit.
 template <typename E>
-int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int64_t b, int j,
-                 void* values, int64_t* indices, void* ws, hipStream_t stream);
+int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
+                 int64_t* indices, void* ws, hipStream_t stream);
 
 }  // namespace stream
 }  // namespace atk

@@ -60,29 +60,33 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
   constexpr int VF = full_vec((int)sizeof(raw_t));
   const int rc = pl.vec > 1 ? launch_w<E, J, VF>(pl, x, out, g, rows, stream)
                             : launch_w<E, J, 1>(pl, x, out, g, rows, stream);
-  if (rc != ATK_OK || pl.slabs == 1) return rc;
-  const int64_t blocks_per_row = (g.b + kWave - 1) / kWave;
+  if (rc != ATK_OK || !pl.merge) return rc;
+  const int64_t b = pl.width / pl.fold;  // buckets
+  uint32_t cb = kWave;                   // buckets per workgroup: a power of two, no more than needed
+  while (cb > 1 && (int64_t)(cb / 2) >= b) cb /= 2;
+  const int64_t blocks_per_row = (b + cb - 1) / cb;
   if (blocks_per_row * rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)),
-                     dim3(kWave * kMergeWaves), 0,
-                     stream, (const raw_t*)out.part_values, (const uint32_t*)out.part_pos, g.b, pl.slabs,
-                     blocks_per_row, out.values, out.indices);
+                     dim3(kMergeThreads), 0,
+                     stream, x, g.row_stride, (const raw_t*)out.part_values, (const uint32_t*)out.part_pos,
+                     b, pl.fold, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
 template <typename E>
-int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int64_t b, int j,
+int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j,
                  void* values, int64_t* indices, void* ws, hipStream_t stream) {
   using raw_t = typename E::raw_t;
   Geom g;
-  g.row_stride = row_stride; g.b = b;
+  g.row_stride = row_stride; g.b = pl.width;
   g.full_rows = pl.full_rows; g.rem = pl.rem; g.pad_tail = pl.pad_tail;
   g.slabs = pl.slabs; g.slab_len = pl.slab_len; g.col_tiles = pl.col_tiles;
+  g.fold = pl.merge ? 1u : pl.fold;
   Sink<raw_t> out;
   out.values = static_cast<raw_t*>(values); out.indices = indices;
   unsigned char* base = static_cast<unsigned char*>(ws);
-  out.part_values = pl.slabs > 1 ? reinterpret_cast<raw_t*>(base + pl.part_values_off) : nullptr;
-  out.part_pos = pl.slabs > 1 ? reinterpret_cast<uint32_t*>(base + pl.part_pos_off) : nullptr;
+  out.part_values = pl.merge ? reinterpret_cast<raw_t*>(base + pl.part_values_off) : nullptr;
+  out.part_pos = pl.merge ? reinterpret_cast<uint32_t*>(base + pl.part_pos_off) : nullptr;
   const raw_t* xs = static_cast<const raw_t*>(x);
   switch (j) {
     case 1: return launch_j<E, 1>(pl, xs, out, g, rows, stream);
@@ -94,8 +98,8 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
 }
 
 #define ATK_INSTANTIATE_STREAM(DT)                                                          \
-  template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int64_t, \
-                                      int, void*, int64_t*, void*, hipStream_t);
+  template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int, void*, \
+                                      int64_t*, void*, hipStream_t);
 
 }  // namespace stream
 }  // namespace atk

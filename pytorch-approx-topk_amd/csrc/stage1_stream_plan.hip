@@ -12,6 +12,9 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 constexpr int64_t kTargetWaves = 1024;
 // Sub-rows worth giving to one wave before a row is also cut into slabs.
 constexpr int64_t kSlabRun = 16;
+// Buckets at least this long are folded when they do not fill a column tile;
+// below, merging the folded columns costs more than the idle lanes.
+constexpr int64_t kFoldMinLength = 128;
 }  // namespace
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned) {
@@ -22,17 +25,33 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   const int es = elem_bytes(dtype);
   if (!es) return pl;
   const int64_t b = k0 / j;
-  const int64_t full = n / b;
-  if (full < j || full > 0xfffffffell || b > 0x7fffffffll) return pl;
-  pl.full_rows = (uint32_t)full;
-  pl.rem = (uint32_t)(n - full * b);
-  pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
+  const int64_t length = n / b;  // elements every bucket has
+  if (length < j || length > 0xfffffffell || b > 0x7fffffffll) return pl;
   const int vf = full_vec(es);
-  pl.vec = (aligned && b % vf == 0) ? vf : 1;
+
+  // Few buckets: scan `fold` sub-rows side by side so that the lanes of a wave
+  // are all busy (the largest fold that fits one column tile and keeps 16-byte
+  // loads possible); each bucket is put back together by the scanning workgroup
+  // or, when the row is also cut into slabs, by the merge kernel.
+  int64_t fold = 1;
+  {
+    const int v = aligned ? vf : 1;
+    int64_t f = (int64_t)kWave * v / b;
+    while (f > 1 && (b * f) % v != 0) --f;
+    if (f > 1 && length >= kFoldMinLength && n / (b * f) >= j) fold = f;
+  }
+  pl.fold = (uint32_t)fold;
+  const int64_t width = b * fold;
+  pl.width = width;
+  const int64_t full = n / width;
+  pl.full_rows = (uint32_t)full;
+  pl.rem = (uint32_t)(n - full * width);
+  pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
+  pl.vec = (aligned && width % vf == 0) ? vf : 1;
   pl.packed = (dtype == ATK_F16 || dtype == ATK_BF16 || dtype == ATK_I16) && full <= kPackedMaxSubRow;
 
   const int64_t tile_cols = (int64_t)kWave * pl.vec;
-  pl.col_tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
+  pl.col_tiles = (uint32_t)((width + tile_cols - 1) / tile_cols);
 
   // Waves per workgroup.  Wave 0's serial work per column is its own run,
   // full/w pushes, plus (w-1)*j pushes to fold the other waves' queues.  Take
@@ -71,8 +90,10 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
     const int64_t run = full / pl.waves;
     if ((run == 4 || run == 8) && run >= j) pl.run = (int)run;
   }
-  if (pl.slabs > 1) {
-    const size_t entries = (size_t)rows * pl.slabs * (size_t)k0;
+  // a folded row that one workgroup scans alone is merged by that workgroup
+  pl.merge = pl.slabs > 1;
+  if (pl.merge) {
+    const size_t entries = (size_t)rows * pl.slabs * (size_t)width * (size_t)j;
     pl.part_values_off = 0;
     pl.part_pos_off = align_up(entries * es, 256);
     pl.ws_bytes = pl.part_pos_off + align_up(entries * sizeof(uint32_t), 256);
@@ -105,7 +126,7 @@ int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_str
   if (pl.ws_bytes && (!ws || ws_bytes < pl.ws_bytes || (uintptr_t)ws % 16 != 0)) return ATK_ERR_WORKSPACE;
   int rc = ATK_ERR_DTYPE;
   ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
-                   rc = stream::launch_typed<E>(pl, x, rows, row_stride, k0 / j, j, values, indices, ws,
+                   rc = stream::launch_typed<E>(pl, x, rows, row_stride, j, values, indices, ws,
                                                 stream));
   return rc;
 }

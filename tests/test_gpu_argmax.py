@@ -70,3 +70,13 @@ def test_k_larger_than_n_and_neg_inf():
             ev, ei = oracle.bucketed_argmax(x, k, 1, interleaved)
             av, ai = topk_triton(x.cuda(), k=k, dim=1, interleaved=interleaved)
             assert_same(av, ai, ev, ei, f"k={k} interleaved={interleaved}")
+
+
+@pytest.mark.parametrize("n,k", [(65536, 64), (50000, 48), (40001, 10), (1 << 20, 1), (4096, 16), (4001, 12)])
+def test_few_long_buckets(n, k):
+    from approx_topk.experimental.bucketed_argmax import topk_triton
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randn(3, n, generator=g)
+    ev, ei = oracle.bucketed_argmax(x, k, 1, True)
+    av, ai = topk_triton(x.cuda(), k=k, dim=1, interleaved=True)
+    assert_same(av, ai, ev, ei, f"n={n} k={k}")

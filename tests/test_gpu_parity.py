@@ -309,3 +309,61 @@ def test_fused_config3_and_config4_full_shapes():
     v, i = _run(x4, 64, -1, j=1, k_mult=8)
     ev, ei = oracle_topk(x4, 64, -1, j=1, k_mult=8)
     assert_same(v, i, ev, ei, "C4")
+
+
+# ---- few, long buckets: the row is scanned several sub-rows side by side and a merge follows ----
+
+@pytest.mark.parametrize("rows,n,k,j", [
+    (32, 65536, 64, 1), (32, 65536, 64, 2), (128, 65536, 64, 4),   # the benchmark sweep's k = 64 shapes
+    (5, 40000, 10, 1),       # 10 buckets: fold 24, 60 lanes busy
+    (3, 30011, 30, 3),       # ragged row, three entries per bucket
+    (2, 70000, 7, 1),        # bucket count not a multiple of the vector width
+    (1, 1 << 22, 4, 4),      # one bucket: exact top-4 of a long row, many slabs
+    (1, (1 << 20) + 13, 1, 1),
+    (3, 20000, 8, 4), (3, 20000, 6, 3),
+    # short enough rows that the scanning workgroup merges the folded columns itself
+    (6, 4096, 16, 1), (6, 4099, 12, 2), (6, 2048, 12, 3), (130, 8192, 64, 4), (3, 5000, 7, 1), (2, 3000, 1, 1),
+])
+def test_few_long_buckets(rows, n, k, j):
+    _check(cpu_randn((rows, n), n + k + j), k, -1, j=j)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("j,k_mult", [(1, 1), (2, 2), (3, 1), (4, 1)])
+@pytest.mark.parametrize("n", [50001, 3001])
+def test_few_long_buckets_all_dtypes_with_ties(dtype, j, k_mult, n):
+    g = torch.Generator().manual_seed(23 + j)
+    shape = (6, n)
+    if dtype.is_floating_point:
+        x = torch.randint(-9, 10, shape, generator=g).to(dtype) / 4
+    elif dtype == torch.uint8:
+        x = torch.randint(0, 19, shape, generator=g).to(dtype)
+    else:
+        x = torch.randint(-9, 10, shape, generator=g).to(dtype)
+    _check(x, 12, -1, j=j, k_mult=k_mult)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("n", [40000, 4100])
+def test_few_long_buckets_special_values(dtype, n):
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn((6, n), generator=g).to(dtype)
+    specials = torch.tensor([float("nan"), float("inf"), -float("inf"), 0.0, -0.0]).to(dtype)
+    for r in range(0, 6, 2):
+        sel = torch.randint(0, n, (500,), generator=g)
+        x[r, sel] = specials[torch.randint(0, 5, (500,), generator=g)]
+    for j, km in [(1, 1), (2, 1), (4, 2)]:
+        _check(x, 16, -1, j=j, k_mult=km)
+
+
+def test_few_long_buckets_unaligned_rows():
+    x = cpu_randn((4, 30001), 77)            # odd row pitch: no 16-byte loads
+    _check(x, 16, -1, j=2)
+    wide = cpu_randn((4, 30016), 78)
+    v, i = _topk()(wide.cuda()[:, 3:30003], 20, -1, j=2)   # misaligned base pointer, pitch > n
+    ev, ei = oracle_topk(wide[:, 3:30003].contiguous(), 20, -1, j=2)
+    assert_same(v, i, ev, ei, "misaligned view")
+    small = cpu_randn((4, 4112), 79)
+    v, i = _topk()(small.cuda()[:, 3:4103], 20, -1, j=2)
+    ev, ei = oracle_topk(small[:, 3:4103].contiguous(), 20, -1, j=2)
+    assert_same(v, i, ev, ei, "misaligned view, short rows")
