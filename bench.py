@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the headline kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
 # copy of known size (profiles/stream_kernel_f32_j2_c2_hbm_traffic.md); None for other workloads.
-MEASURED_TRAFFIC_BYTES = {"C2": 637_638_750}
+MEASURED_TRAFFIC_BYTES = {"C2": 637_602_610}
 
 # name -> (rows, n, dtype, k, j, k_mult, seed)
 CONFIGS = {
