@@ -52,6 +52,9 @@ int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64
   const int rc = atk::launch_stage1_stream(x, rows, n, row_stride, k0, j, layout, dtype, values,
                                            indices, ws, ws_bytes, stream, &handled);
   if (handled || rc != ATK_OK) return rc;
+  const int rc2 = atk::launch_stage1_contig(x, rows, n, row_stride, k0, j, layout, dtype, values, indices,
+                                            stream, &handled);
+  if (handled || rc2 != ATK_OK) return rc2;
   return atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout, dtype, values,
                                             indices, stream);
 }

@@ -1,0 +1,249 @@
+// Stage 1 for the contiguous layouts (every bucket a run of adjacent elements).
+//
+// Reading a bucket front to back with one lane per bucket puts a whole bucket
+// length between the addresses of neighbouring lanes.  Here a workgroup instead
+// copies a span of whole buckets from the row into LDS with coalesced 16-byte
+// loads and scans it from there: each of its 256 threads walks one *piece* of a
+// bucket (at most 32 adjacent elements; 16 for 8-byte types) with a J-entry
+// queue in registers, the P = 2^k threads that share a bucket combine their
+// queues through LDS with the merge network of stage1_stream.h under the full
+// order (value, then lower index), and the first of them writes the bucket's J
+// entries.  A workgroup covers 256 / P adjacent buckets.  A bucket longer than
+// 256 pieces takes a workgroup of its own, which goes through it in chunks of
+// 256 pieces; a thread's queue then lives across the chunks (its pieces come
+// in increasing position, so a newcomer still only displaces what it beats
+// strictly).
+//
+// LDS placement.  Element i of the span sits at i + i/32 words' worth of
+// elements (one 4-byte word of padding per 32 elements): the 4-byte writes of a
+// 16-byte pack stay adjacent, and threads that read with a stride of one piece
+// (any length, powers of two included) spread over the banks.
+//
+// Values.  Floating-point elements are compared in IEEE form, and the copy into
+// LDS tests every element for NaN; a workgroup that finds one starts over with
+// the integer order keys of atk_device.h (NaN above +inf, all NaN equal).
+// Positions >= n (the padded arg-max layout) hold the pad element.
+#pragma once
+
+#include "stage1_stream.h"
+
+namespace atk {
+namespace contig {
+
+using stream::Cmp;
+using stream::MergeWord;
+using stream::Pack;
+
+constexpr int kThreads = 256;
+
+// Longest piece one thread scans.
+__host__ __device__ constexpr int max_piece(int elem_size) { return elem_size == 8 ? 16 : 32; }
+// LDS elements of padding per 32 elements: one 4-byte word's worth.
+__host__ __device__ constexpr int pad_elems(int elem_size) { return elem_size >= 4 ? 1 : 4 / elem_size; }
+
+struct Geom {
+  int64_t row_stride;    // elements between rows
+  int64_t n;             // real elements per row; positions beyond hold the pad element
+  uint32_t b;            // buckets per row
+  uint32_t m;            // elements per bucket (balanced layout: of the shorter buckets)
+  uint32_t r;            // balanced layout: the first r buckets hold m + 1 elements
+  uint32_t pieces_log2;  // log2 of P, the threads per bucket
+  uint32_t trip;         // the longest piece of any thread
+  uint32_t chunks;       // > 1: one bucket per workgroup, scanned in that many chunks
+  uint32_t groups;       // workgroups per row
+};
+
+// How a thread's queue holds values: in compare form (fast; no NaN may be
+// present) or as order keys (exact).
+template <typename E> struct CmpForm {
+  using T = typename Cmp<E>::cmp_t;
+  using M = MergeWord<E>;
+  __device__ static __forceinline__ T conv(typename E::raw_t raw) { return Cmp<E>::from_raw(raw); }
+  __device__ static __forceinline__ typename M::word_t word(T v, uint32_t p) { return M::make(Cmp<E>::to_raw(v), p); }
+};
+template <typename E> struct KeyForm {
+  using T = typename E::key_t;
+  using M = MergeWord<E>;
+  __device__ static __forceinline__ T conv(typename E::raw_t raw) { return E::key(raw); }
+  __device__ static __forceinline__ typename M::word_t word(T v, uint32_t p) { return M::from_key(v, p); }
+};
+
+template <typename E> __device__ __forceinline__ uint32_t lds_slot(uint32_t i) {
+  return i + (i >> 5) * (uint32_t)pad_elems((int)sizeof(typename E::raw_t));
+}
+
+// One pass over the workgroup's buckets in form F.  Returns false, having
+// written nothing, when F cannot order the data (a NaN in compare form).
+template <typename E, int J, int V, typename F>
+__device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict__ xr,
+                                             typename E::raw_t* __restrict__ values,
+                                             int64_t* __restrict__ indices, int64_t row, uint32_t group,
+                                             const Geom& g, unsigned char* lds) {
+  using raw_t = typename E::raw_t;
+  using T = typename F::T;
+  using M = typename F::M;
+  using word_t = typename M::word_t;
+  constexpr int N = J == 3 ? 4 : J;
+  constexpr bool kScreen = Cmp<E>::has_nan && std::is_same<F, CmpForm<E>>::value;
+  constexpr uint32_t kChunk = kThreads * max_piece((int)sizeof(raw_t));
+  raw_t* data = reinterpret_cast<raw_t*>(lds);
+
+  const uint32_t t = threadIdx.x;
+  const uint32_t pieces = 1u << g.pieces_log2;
+  const uint32_t per_group = kThreads >> g.pieces_log2;  // buckets per workgroup
+  const uint32_t c0 = group * per_group;
+  const uint32_t c = c0 + (t >> g.pieces_log2);
+  const uint32_t piece = t & (pieces - 1);
+  const bool has = c < g.b;
+  auto start_of = [&](uint32_t bucket) -> uint32_t { return bucket * g.m + (bucket < g.r ? bucket : g.r); };
+  const uint32_t start = start_of(c);
+  const uint32_t len = g.m + (c < g.r ? 1u : 0u);
+  const uint32_t c1 = c0 + per_group < g.b ? c0 + per_group : g.b;
+
+  T q[J];
+  uint32_t pos[J];
+  for (uint32_t it = 0; it < g.chunks; ++it) {
+    // the span this round: all the workgroup's buckets, or one chunk of its only bucket
+    uint32_t e0, e1;
+    if (g.chunks == 1) {
+      e0 = start_of(c0);
+      e1 = start_of(c1);
+    } else {
+      e0 = start_of(c0) + it * kChunk;
+      const uint32_t end = start_of(c0) + g.m + (c0 < g.r ? 1u : 0u);
+      e1 = e0 + kChunk < end ? e0 + kChunk : end;
+    }
+    const uint32_t a0 = e0 & ~(uint32_t)(V - 1);  // packs are aligned in the row
+    if (it != 0) __syncthreads();                 // the last round's reads are done
+
+    bool nan = false;
+    const uint32_t packs = (e1 - a0 + V - 1) / V;
+    for (uint32_t pk = t; pk < packs; pk += kThreads) {
+      const uint32_t at = a0 + pk * V;
+      Pack<raw_t, V> got;
+      if ((int64_t)at + V <= g.n) {
+        got = stream::load_pack<raw_t, V>(xr + at);
+      } else {
+        ATK_STATIC_FOR(e, V) { got.e[e] = (int64_t)at + e < g.n ? xr[at + e] : E::pad_raw; } ATK_STATIC_END;
+      }
+      if constexpr (kScreen) {
+        ATK_STATIC_FOR(h, V / 2) {
+          nan |= __builtin_isunordered(F::conv(got.e[2 * h]), F::conv(got.e[2 * h + 1]));
+        } ATK_STATIC_END;
+        if constexpr (V % 2 != 0) nan |= __builtin_isunordered(F::conv(got.e[V - 1]), F::conv(got.e[V - 1]));
+      }
+      const uint32_t slot = lds_slot<E>(pk * V);  // the V elements of a pack stay adjacent
+      if constexpr (V * sizeof(raw_t) % 4 == 0) {
+        uint32_t words[V * sizeof(raw_t) / 4];
+        __builtin_memcpy(words, &got, sizeof(words));
+        uint32_t* dst = reinterpret_cast<uint32_t*>(data + slot);
+        ATK_STATIC_FOR(w, (int)(V * sizeof(raw_t) / 4)) { dst[w] = words[w]; } ATK_STATIC_END;
+      } else {
+        ATK_STATIC_FOR(e, V) { data[slot + e] = got.e[e]; } ATK_STATIC_END;
+      }
+    }
+    if constexpr (kScreen) {
+      if (__syncthreads_or(nan)) return false;
+    } else {
+      __syncthreads();
+    }
+
+    // this thread's piece [lo, hi) of its bucket
+    uint32_t lo, hi;
+    if (g.chunks == 1) {
+      lo = (uint32_t)(((uint64_t)len * piece) >> g.pieces_log2);
+      hi = (uint32_t)(((uint64_t)len * (piece + 1)) >> g.pieces_log2);
+    } else {
+      lo = it * kChunk + piece * (uint32_t)max_piece((int)sizeof(raw_t));
+      hi = lo + (uint32_t)max_piece((int)sizeof(raw_t));
+      lo = lo < len ? lo : len;
+      hi = hi < len ? hi : len;
+    }
+    if (has) {
+      const uint32_t count = hi - lo;
+      const uint32_t first = start + lo;  // position in the row
+      const uint32_t li = first - a0;     // position in the span
+      uint32_t s = 0;
+      if (it == 0) {  // every piece of the first round holds at least J elements
+        ATK_STATIC_FOR(u, J) {
+          stream::push<T, J, u>(q, pos, F::conv(data[lds_slot<E>(li + u)]), first + u);
+        } ATK_STATIC_END;
+        s = J;
+      }
+#pragma unroll 4
+      for (; s < g.trip; ++s) {
+        const bool valid = s < count;
+        const T v = F::conv(data[lds_slot<E>(li + (valid ? s : 0u))]);
+        stream::push<T, J, J>(q, pos, valid ? v : q[0], first + s);  // q[0] beats nothing
+      }
+    }
+  }
+
+  // combine the pieces of every bucket
+  word_t acc[N], in[N];
+  ATK_STATIC_FOR(sl, N) { acc[sl] = M::empty(); in[sl] = M::empty(); } ATK_STATIC_END;
+  if (has) {
+    ATK_STATIC_FOR(sl, J) { acc[N - J + sl] = F::word(q[sl], pos[sl]); } ATK_STATIC_END;
+  }
+  if (pieces > 1) {
+    __syncthreads();  // the span is no longer read: its LDS now carries the queues
+    word_t* lists = reinterpret_cast<word_t*>(lds);  // [N][kThreads]
+    for (uint32_t half = pieces / 2; half >= 1; half /= 2) {
+      if (piece >= half && piece < 2 * half) {
+        ATK_STATIC_FOR(sl, N) { lists[sl * kThreads + t] = acc[sl]; } ATK_STATIC_END;
+      }
+      __syncthreads();
+      if (piece < half) {
+        ATK_STATIC_FOR(sl, N) { in[sl] = lists[sl * kThreads + t + half]; } ATK_STATIC_END;
+        stream::merge_best<M, N>(acc, in);
+      }
+    }
+  }
+  if (has && piece == 0) {
+    const int64_t o = (row * g.b + c) * J;
+    ATK_STATIC_FOR(sl, J) {
+      const uint32_t p = M::pos(acc[N - J + sl]);
+      values[o + sl] = (int64_t)p < g.n ? xr[p] : E::pad_raw;
+      indices[o + sl] = p;
+    } ATK_STATIC_END;
+  }
+  return true;
+}
+
+// E: element traits; J: entries kept per bucket; V: elements per load (16
+// bytes' worth when the row allows it, else 1).
+template <typename E, int J, int V>
+__global__ __launch_bounds__(kThreads) void contig_kernel(const typename E::raw_t* __restrict__ x,
+                                                          typename E::raw_t* __restrict__ values,
+                                                          int64_t* __restrict__ indices, const Geom g) {
+  extern __shared__ __align__(16) unsigned char contig_lds[];
+  const uint32_t row32 = blockIdx.x / g.groups;
+  const uint32_t group = blockIdx.x - row32 * g.groups;
+  const int64_t row = row32;
+  const typename E::raw_t* xr = x + row * g.row_stride;
+  if (scan_buckets<E, J, V, CmpForm<E>>(xr, values, indices, row, group, g, contig_lds)) return;
+  if constexpr (Cmp<E>::has_nan) {
+    __syncthreads();
+    scan_buckets<E, J, V, KeyForm<E>>(xr, values, indices, row, group, g, contig_lds);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+struct Plan {
+  bool ok;
+  int vec;           // V
+  Geom geom;         // row_stride is filled in at launch
+  size_t lds_bytes;  // dynamic LDS per workgroup
+};
+
+// `aligned`: base pointer and row stride allow 16-byte loads.
+Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned);
+
+template <typename E>
+int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
+                 int64_t* indices, hipStream_t stream);
+
+}  // namespace contig
+}  // namespace atk

@@ -1,0 +1,70 @@
+// Host-side planning and dispatch of the contiguous-layout stage-1 kernel.
+#include "stage1_contig.h"
+
+namespace atk {
+namespace contig {
+
+Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned) {
+  Plan pl{};
+  pl.ok = false;
+  if (layout != ATK_BALANCED && layout != ATK_CEIL_CHUNK) return pl;
+  if (rows <= 0 || n <= 0 || k0 <= 0 || j < 1 || j > 4 || k0 % j) return pl;
+  const int es = elem_bytes(dtype);
+  if (!es) return pl;
+  const int64_t b = k0 / j;
+  const int64_t m = layout == ATK_BALANCED ? n / b : (n + b - 1) / b;
+  const int64_t r = layout == ATK_BALANCED ? n - m * b : 0;
+  // every bucket holds at least j elements; positions fit 32 bits
+  if (m < j || b > 0x7fffffffll || (double)b * (double)m + (double)r > 4294967294.0) return pl;
+  const int64_t longest = m + (r > 0 ? 1 : 0);
+  const int64_t piece = max_piece(es);
+
+  Geom& g = pl.geom;
+  g.n = n;
+  g.b = (uint32_t)b;
+  g.m = (uint32_t)m;
+  g.r = (uint32_t)r;
+  uint32_t lg = 0;
+  while (lg < 8 && ((longest + (1ll << lg) - 1) >> lg) > piece) ++lg;
+  g.pieces_log2 = lg;
+  const int64_t per_thread = (longest + (1ll << lg) - 1) >> lg;
+  if (per_thread > piece) {  // lg == 8: a workgroup per bucket, in chunks of 256 pieces
+    g.chunks = (uint32_t)((longest + kThreads * piece - 1) / (kThreads * piece));
+    g.trip = (uint32_t)piece;
+  } else {
+    g.chunks = 1;
+    g.trip = (uint32_t)per_thread;
+  }
+  const int64_t per_group = kThreads >> lg;
+  g.groups = (uint32_t)((b + per_group - 1) / per_group);
+  if (rows * (int64_t)g.groups > 0x7fffffffll) return pl;
+
+  pl.vec = aligned ? stream::full_vec(es) : 1;
+  // LDS: the longest span (whole packs, one element of slack) with its padding, or the queues
+  const int64_t span = (g.chunks > 1 ? kThreads * piece : per_group * longest) + 2 * pl.vec + 2;
+  const size_t data_bytes = (size_t)(span + ((span >> 5) + 1) * pad_elems(es)) * es;
+  const size_t list_bytes = (size_t)4 * kThreads * (es == 8 ? 16 : 8);
+  pl.lds_bytes = ((data_bytes > list_bytes ? data_bytes : list_bytes) + 15) / 16 * 16;
+  if (pl.lds_bytes > 64 * 1024) return pl;
+  pl.ok = true;
+  return pl;
+}
+
+}  // namespace contig
+
+int launch_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                         int layout, int dtype, void* values, int64_t* indices, hipStream_t stream,
+                         bool* handled) {
+  const int es = elem_bytes(dtype);
+  const int vf = es ? stream::full_vec(es) : 1;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && (row_stride % vf == 0);
+  const contig::Plan pl = contig::make_plan(rows, n, k0, j, layout, dtype, aligned);
+  *handled = pl.ok;
+  if (!pl.ok) return ATK_OK;
+  int rc = ATK_ERR_DTYPE;
+  ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
+                   rc = contig::launch_typed<E>(pl, x, rows, row_stride, j, values, indices, stream));
+  return rc;
+}
+
+}  // namespace atk

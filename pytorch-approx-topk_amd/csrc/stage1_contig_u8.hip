@@ -1,0 +1,8 @@
+// Contiguous-layout stage-1 kernel instantiated for one element type.
+#include "stage1_contig_launch.h"
+
+namespace atk {
+namespace contig {
+ATK_INSTANTIATE_CONTIG(ATK_U8)
+}  // namespace contig
+}  // namespace atk

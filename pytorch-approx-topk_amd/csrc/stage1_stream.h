@@ -577,6 +577,9 @@ template <typename E, bool WIDE = (E::key_bits > 32)> struct MergeWord {
   __device__ static __forceinline__ word_t make(typename E::raw_t raw, uint32_t p) {
     return ((uint64_t)E::key(raw) << 32) | (uint64_t)(0xffffffffu - p);
   }
+  __device__ static __forceinline__ word_t from_key(typename E::key_t key, uint32_t p) {
+    return ((uint64_t)key << 32) | (uint64_t)(0xffffffffu - p);
+  }
   __device__ static __forceinline__ word_t empty() { return 0; }
   __device__ static __forceinline__ bool better(word_t a, word_t b) { return a > b; }
   __device__ static __forceinline__ uint32_t pos(word_t w) { return 0xffffffffu - (uint32_t)w; }
@@ -586,6 +589,9 @@ template <typename E> struct MergeWord<E, true> {
   struct word_t { uint64_t key; uint32_t npos; uint32_t unused; };
   __device__ static __forceinline__ word_t make(typename E::raw_t raw, uint32_t p) {
     return word_t{E::key(raw), 0xffffffffu - p, 0u};
+  }
+  __device__ static __forceinline__ word_t from_key(uint64_t key, uint32_t p) {
+    return word_t{key, 0xffffffffu - p, 0u};
   }
   __device__ static __forceinline__ word_t empty() { return word_t{0, 0, 0}; }
   __device__ static __forceinline__ bool better(const word_t& a, const word_t& b) {

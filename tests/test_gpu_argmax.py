@@ -80,3 +80,15 @@ def test_few_long_buckets(n, k):
     ev, ei = oracle.bucketed_argmax(x, k, 1, True)
     av, ai = topk_triton(x.cuda(), k=k, dim=1, interleaved=True)
     assert_same(av, ai, ev, ei, f"n={n} k={k}")
+
+
+@pytest.mark.parametrize("n,k", [(65536, 64), (50000, 48), (40001, 10), (1 << 20, 1), (4096, 16), (4001, 12), (100, 64), (5000, 4999)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.int64])
+def test_contiguous_chunks(n, k, dtype):
+    from approx_topk.experimental.bucketed_argmax import topk_triton
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randn(3, n, generator=g)
+    x = (x * 1000).to(dtype) if not dtype.is_floating_point else x.to(dtype)
+    ev, ei = oracle.bucketed_argmax(x, k, 1, False)
+    av, ai = topk_triton(x.cuda(), k=k, dim=1, interleaved=False)
+    assert_same(av, ai, ev, ei, f"n={n} k={k}")

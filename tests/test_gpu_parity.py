@@ -367,3 +367,43 @@ def test_few_long_buckets_unaligned_rows():
     v, i = _topk()(small.cuda()[:, 3:4103], 20, -1, j=2)
     ev, ei = oracle_topk(small[:, 3:4103].contiguous(), 20, -1, j=2)
     assert_same(v, i, ev, ei, "misaligned view, short rows")
+
+
+# ---- contiguous buckets: spans of whole buckets staged in LDS, pieces per thread, long buckets in chunks ----
+
+@pytest.mark.parametrize("rows,n,k,j", [
+    (130, 4096, 128, 1),     # 32-element buckets, one thread each
+    (7, 4100, 100, 2),       # 82/83-element buckets: four threads per bucket, ragged
+    (3, 100003, 4, 2),       # two buckets of 50001/50002: a workgroup per bucket, seven chunks
+    (2, 70000, 3, 3),        # one bucket, three entries
+    (4, 9000, 1, 1),         # one bucket a little over one chunk
+    (5, 2 * 8192 + 5, 2, 1), # buckets of 8194/8195: the last chunk holds two or three elements
+    (3, 5000, 1250, 2), (3, 70001, 4096, 4), (2, 333, 333, 1), (2, 1024, 512, 2),
+])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.float64, torch.int8])
+def test_contiguous_buckets(rows, n, k, j, dtype):
+    x = cpu_randn((rows, n), n + k + j)
+    x = (x * 40).to(dtype) if not dtype.is_floating_point else x.to(dtype)
+    _check(x, k, -1, j=j, interleaved=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("n,k", [(40000, 16), (4100, 64), (100000, 2)])
+def test_contiguous_buckets_special_values(dtype, n, k):
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn((6, n), generator=g).to(dtype)
+    specials = torch.tensor([float("nan"), float("inf"), -float("inf"), 0.0, -0.0]).to(dtype)
+    for r in range(0, 6, 2):
+        sel = torch.randint(0, n, (500,), generator=g)
+        x[r, sel] = specials[torch.randint(0, 5, (500,), generator=g)]
+    for j, km in [(1, 1), (2, 1), (2, 2)]:
+        _check(x, k, -1, j=j, k_mult=km, interleaved=False)
+
+
+def test_contiguous_buckets_unaligned_rows():
+    x = cpu_randn((4, 30001), 81)
+    _check(x, 16, -1, j=2, interleaved=False)
+    wide = cpu_randn((4, 30016), 82)
+    v, i = _topk()(wide.cuda()[:, 3:30003], 20, -1, j=2, interleaved=False)
+    ev, ei = oracle_topk(wide[:, 3:30003].contiguous(), 20, -1, j=2, interleaved=False)
+    assert_same(v, i, ev, ei, "misaligned view")
