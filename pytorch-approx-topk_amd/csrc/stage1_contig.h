@@ -35,6 +35,7 @@ using stream::MergeWord;
 using stream::Pack;
 
 constexpr int kThreads = 256;
+constexpr int kLoads = 8;  // loads one thread keeps in flight while a span is copied
 
 // Longest piece one thread scans.
 __host__ __device__ constexpr int max_piece(int elem_size) { return elem_size == 8 ? 16 : 32; }
@@ -49,6 +50,7 @@ struct Geom {
   uint32_t r;            // balanced layout: the first r buckets hold m + 1 elements
   uint32_t pieces_log2;  // log2 of P, the threads per bucket
   uint32_t trip;         // the longest piece of any thread
+  uint32_t sure;         // the shortest piece of any thread (one chunk; chunks but the last are full)
   uint32_t chunks;       // > 1: one bucket per workgroup, scanned in that many chunks
   uint32_t groups;       // workgroups per row
 };
@@ -118,14 +120,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
 
     bool nan = false;
     const uint32_t packs = (e1 - a0 + V - 1) / V;
-    for (uint32_t pk = t; pk < packs; pk += kThreads) {
-      const uint32_t at = a0 + pk * V;
-      Pack<raw_t, V> got;
-      if ((int64_t)at + V <= g.n) {
-        got = stream::load_pack<raw_t, V>(xr + at);
-      } else {
-        ATK_STATIC_FOR(e, V) { got.e[e] = (int64_t)at + e < g.n ? xr[at + e] : E::pad_raw; } ATK_STATIC_END;
-      }
+    auto park = [&](uint32_t pk, const Pack<raw_t, V>& got) __attribute__((always_inline)) {
       if constexpr (kScreen) {
         ATK_STATIC_FOR(h, V / 2) {
           nan |= __builtin_isunordered(F::conv(got.e[2 * h]), F::conv(got.e[2 * h + 1]));
@@ -141,6 +136,27 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
       } else {
         ATK_STATIC_FOR(e, V) { data[slot + e] = got.e[e]; } ATK_STATIC_END;
       }
+    };
+    // packs that lie inside the row: kLoads loads in flight per thread
+    const int64_t inside = (g.n - (int64_t)a0) / V;
+    const uint32_t whole = inside <= 0 ? 0u : (inside < (int64_t)packs ? (uint32_t)inside : packs);
+    for (uint32_t base = 0; base < whole; base += kThreads * kLoads) {
+      Pack<raw_t, V> got[kLoads];
+      ATK_STATIC_FOR(u, kLoads) {
+        const uint32_t pk = base + u * kThreads + t;
+        got[u] = stream::load_pack<raw_t, V>(xr + a0 + (size_t)(pk < whole ? pk : whole - 1) * V);
+      } ATK_STATIC_END;
+      ATK_STATIC_FOR(u, kLoads) {
+        const uint32_t pk = base + u * kThreads + t;
+        if (pk < whole) park(pk, got[u]);
+      } ATK_STATIC_END;
+    }
+    // packs that reach past the row's end: the pad element beyond it
+    for (uint32_t pk = whole + t; pk < packs; pk += kThreads) {
+      const uint32_t at = a0 + pk * V;
+      Pack<raw_t, V> got;
+      ATK_STATIC_FOR(e, V) { got.e[e] = (int64_t)at + e < g.n ? xr[at + e] : E::pad_raw; } ATK_STATIC_END;
+      park(pk, got);
     }
     if constexpr (kScreen) {
       if (__syncthreads_or(nan)) return false;
@@ -170,7 +186,12 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
         } ATK_STATIC_END;
         s = J;
       }
+      // every piece holds `sure` elements; only the few after that need a check
+      const uint32_t sure = g.chunks == 1 ? g.sure : (it + 1 < g.chunks ? g.trip : 0u);
 #pragma unroll 4
+      for (; s < sure; ++s) {
+        stream::push<T, J, J>(q, pos, F::conv(data[lds_slot<E>(li + s)]), first + s);
+      }
       for (; s < g.trip; ++s) {
         const bool valid = s < count;
         const T v = F::conv(data[lds_slot<E>(li + (valid ? s : 0u))]);

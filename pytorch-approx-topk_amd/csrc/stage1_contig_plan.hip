@@ -34,6 +34,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   } else {
     g.chunks = 1;
     g.trip = (uint32_t)per_thread;
+    g.sure = (uint32_t)(m >> lg);
   }
   const int64_t per_group = kThreads >> lg;
   g.groups = (uint32_t)((b + per_group - 1) / per_group);
