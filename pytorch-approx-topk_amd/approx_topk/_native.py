@@ -83,8 +83,24 @@ def require_gpu(xs: torch.Tensor) -> None:
             "the HIP kernels have no CPU path")
 
 
-def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+def _stream(device: torch.device) -> int:
+    """Raw handle of the current stream of `device` (no Python stream object is built)."""
+    return torch._C._cuda_getCurrentRawStream(device.index)
+
+
+class _on_device:
+    """Makes `device` current for a native call; free when it already is."""
+
+    def __init__(self, device: torch.device):
+        self.guard = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
 
 
 def rows_view(xs: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
@@ -119,12 +135,12 @@ def stage1(xs: torch.Tensor, k0: int, j: int, layout: int) -> tuple[torch.Tensor
     shape = list(xs.shape[:-1]) + [k0]
     values = torch.empty(shape, dtype=xs.dtype, device=xs.device)
     indices = torch.empty(shape, dtype=torch.int64, device=xs.device)
-    with torch.cuda.device(xs.device):
+    with _on_device(xs.device):
         need = L.atk_stage1_workspace_bytes(rows, n, k0, j, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
         check(L.atk_stage1(xs.data_ptr(), rows, n, step, k0, j, layout, code,
                            values.data_ptr(), indices.data_ptr(),
-                           ws.data_ptr() if ws is not None else None, need, _stream()))
+                           ws.data_ptr() if ws is not None else None, need, _stream(xs.device)))
     return values, indices
 
 
@@ -140,12 +156,12 @@ def select(cand_values: torch.Tensor, cand_indices: torch.Tensor, k: int,
     shape = list(cv.shape[:-1]) + [k]
     values = torch.empty(shape, dtype=cv.dtype, device=cv.device)
     indices = torch.empty(shape, dtype=torch.int64, device=cv.device)
-    with torch.cuda.device(cv.device):
+    with _on_device(cv.device):
         need = L.atk_select_workspace_bytes(rows, k0, k, code)
         ws = torch.empty(need, dtype=torch.uint8, device=cv.device) if need else None
         check(L.atk_select(cv.data_ptr(), ci.data_ptr(), rows, k0, k, index_bound, code,
                            values.data_ptr(), indices.data_ptr(),
-                           ws.data_ptr() if ws is not None else None, need, _stream()))
+                           ws.data_ptr() if ws is not None else None, need, _stream(cv.device)))
     return values, indices
 
 
@@ -158,10 +174,10 @@ def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int) -> tuple[torch.
     shape = list(xs.shape[:-1]) + [k]
     values = torch.empty(shape, dtype=xs.dtype, device=xs.device)
     indices = torch.empty(shape, dtype=torch.int64, device=xs.device)
-    with torch.cuda.device(xs.device):
+    with _on_device(xs.device):
         need = L.atk_topk_workspace_bytes(rows, n, k0, j, k, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
         check(L.atk_topk(xs.data_ptr(), rows, n, step, k0, j, k, layout, code,
                          values.data_ptr(), indices.data_ptr(),
-                         ws.data_ptr() if ws is not None else None, need, _stream()))
+                         ws.data_ptr() if ws is not None else None, need, _stream(xs.device)))
     return values, indices
