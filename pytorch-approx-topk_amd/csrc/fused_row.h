@@ -43,7 +43,7 @@ __global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
   constexpr int U = PACKED ? (V * J <= 8 ? 8 : 4) : (J <= 2 ? 8 : 4);
 
   extern __shared__ __align__(16) unsigned char dyn_lds[];
-  __shared__ select::Shared sh;
+  __shared__ select::SharedT<4> sh;  // four histogram copies: four workgroups of C3's shape fit one CU's LDS
   // Candidates, and the hand-over area of the waves that share a tile: behind
   // the candidates, or (hand_off == 0, single round only) on top of them, in
   // which case a barrier separates the last fold from the first candidate.

@@ -30,16 +30,23 @@ static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, 
   return launch_packed<E, J, V, MAXW, pos_t, false>(pl, x, rows, g, k0, k, values, indices, stream);
 }
 
+template <typename E, int J, int VF>
+static int launch_v(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
+                    uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+  if (pl.waves > 8) return ATK_ERR_ARG;  // the planner never asks for more
+  return pl.pos16 ? launch_one<E, J, VF, 8, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
+                  : launch_one<E, J, VF, 8, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
+}
+
 template <typename E, int J>
 static int launch_j(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                     uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
   constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
-  if (pl.waves <= 8) {
-    return pl.pos16 ? launch_one<E, J, VF, 8, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
-                    : launch_one<E, J, VF, 8, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
+  if constexpr (stream::PackedKey<E>::available) {
+    // packed queues may run at half the load width (fewer registers, more workgroups per CU)
+    if (pl.vec == VF / 2) return launch_v<E, J, VF / 2>(pl, x, rows, g, k0, k, values, indices, stream);
   }
-  return pl.pos16 ? launch_one<E, J, VF, 16, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
-                  : launch_one<E, J, VF, 16, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
+  return launch_v<E, J, VF>(pl, x, rows, g, k0, k, values, indices, stream);
 }
 
 template <typename E>

@@ -10,9 +10,10 @@ constexpr int64_t kMinRows = 128;
 // Dynamic LDS a workgroup may use (candidates + hand-over); the select's own
 // block adds about 9 KiB.
 constexpr size_t kLdsBudget = 64 * 1024;
-// Waves per workgroup: 16, or 8 for the element types whose lanes own 8 columns
-// (their queues need the register budget of a smaller workgroup).
-inline uint32_t max_waves(int vec) { return vec <= 4 ? 16u : 8u; }
+// Most waves per workgroup.  Measured over shapes from [4096, 4096] to
+// [256, 65536]: 8 beats 16 (more workgroups per CU, in different phases, and
+// cheaper barriers) and is never far behind 4.
+constexpr uint32_t kMaxWaves = 8;
 }  // namespace
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned) {
@@ -27,13 +28,16 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   const int64_t b = k0 / j;
   const int64_t full = n / b;
   if (full < j || full > 0x7fffffffll) return pl;
-  pl.vec = stream::full_vec(es);
-  if (b % pl.vec) return pl;
   pl.full_rows = (uint32_t)full;
   pl.rem = (uint32_t)(n - full * b);
   pl.pad_tail = 0;
   pl.pos16 = full + 1 <= 0xffff;
   pl.packed = (dtype == ATK_F16 || dtype == ATK_BF16 || dtype == ATK_I16) && full <= stream::kPackedMaxSubRow;
+  pl.vec = stream::full_vec(es);
+  // packed queues at half the load width need about 50 VGPRs instead of 127:
+  // twice the workgroups per CU, which is worth more here than 16-byte loads
+  if (pl.packed) pl.vec /= 2;
+  if (b % pl.vec) return pl;
   const int64_t bound = (full + 1) * b;  // indices are < this
   pl.index_bits = 1;
   while (pl.index_bits < 63 && (1ll << pl.index_bits) < bound) ++pl.index_bits;
@@ -54,7 +58,6 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   // the candidates.
   const int cmp_size = es > 4 ? 8 : 4;
   const int64_t min_run = j > 8 ? j : 8;
-  const uint32_t kMaxWaves = max_waves(pl.vec);
   auto hand_bytes = [&](uint32_t split) {
     const uint32_t waves = pl.tiles * split <= kMaxWaves ? pl.tiles * split : kMaxWaves;
     return (size_t)(waves - waves / split) * pl.vec * j * stream::kWave * (cmp_size + 4);

@@ -20,21 +20,23 @@ namespace select {
 constexpr int kWave = 64;
 constexpr int kMaxWaves = 16;
 
-// Histogram counters are kept in kCopies private copies (lane % kCopies picks
+// Histogram counters are kept in COPIES private copies (lane % kCopies picks
 // one) so that the many candidates sharing a digit -- the top byte of a float
 // key is nearly constant among top-k candidates -- do not serialise on one LDS
 // address; the odd stride spreads equal digits of different copies over banks.
-constexpr int kCopies = 8;
 constexpr int kCopyStride = 257;
 
-struct Shared {
-  uint32_t copies[kCopies * kCopyStride];
+template <int COPIES> struct SharedT {
+  static constexpr int kCopies = COPIES;
+  uint32_t copies[COPIES * kCopyStride];
   uint32_t hist[256];
   uint32_t wave_total[kMaxWaves];
   uint32_t digit;
   uint32_t need;
   uint32_t bin_count;
 };
+using Shared = SharedT<8>;  // the stand-alone select kernel; the fused kernel takes fewer copies to save LDS
+
 
 __device__ __forceinline__ uint32_t lane_id() {
   return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
@@ -47,11 +49,11 @@ __device__ __forceinline__ uint32_t rank_in(uint64_t m) {
 }
 
 // hist[d] = sum of the private copies of bin d
-__device__ __forceinline__ void fold_copies(Shared& sh) {
+template <typename Sh> __device__ __forceinline__ void fold_copies(Sh& sh) {
   for (uint32_t d = threadIdx.x; d < 256; d += blockDim.x) {
     uint32_t total = 0;
 #pragma unroll
-    for (int c = 0; c < kCopies; ++c) total += sh.copies[c * kCopyStride + d];
+    for (int c = 0; c < Sh::kCopies; ++c) total += sh.copies[c * kCopyStride + d];
     sh.hist[d] = total;
   }
 }
@@ -59,8 +61,8 @@ __device__ __forceinline__ void fold_copies(Shared& sh) {
 // Wave 0 scans the 256-bin histogram for the bin holding the `need`-th element,
 // counting from the top bin (FROM_TOP) or from the bottom bin, and publishes
 // the bin, the rank left within it and the bin's population.
-template <bool FROM_TOP>
-__device__ __forceinline__ void find_bin(Shared& sh, uint32_t need) {
+template <bool FROM_TOP, typename Sh>
+__device__ __forceinline__ void find_bin(Sh& sh, uint32_t need) {
   if (threadIdx.x < kWave) {
     const uint32_t lane = threadIdx.x;
     // Lane l owns bins 4l..4l+3.
@@ -93,12 +95,12 @@ __device__ __forceinline__ void find_bin(Shared& sh, uint32_t need) {
 
 // One radix pass: histogram digit `shift` of the values `digit_source(i)` over
 // the candidates with `participates(i)`, then locate the bin of rank `need`.
-template <bool FROM_TOP, typename Participates>
-__device__ __forceinline__ void radix_pass(Shared& sh, uint32_t k0, uint32_t need, Participates digit_or_skip) {
+template <bool FROM_TOP, typename Participates, typename Sh>
+__device__ __forceinline__ void radix_pass(Sh& sh, uint32_t k0, uint32_t need, Participates digit_or_skip) {
   const uint32_t tid = threadIdx.x, nt = blockDim.x;
-  uint32_t* my_copy = &sh.copies[(tid % kCopies) * kCopyStride];
+  uint32_t* my_copy = &sh.copies[(tid % Sh::kCopies) * kCopyStride];
   __syncthreads();
-  for (uint32_t i = tid; i < kCopies * kCopyStride; i += nt) sh.copies[i] = 0;
+  for (uint32_t i = tid; i < Sh::kCopies * kCopyStride; i += nt) sh.copies[i] = 0;
   __syncthreads();
   // four candidates per trip, so that their LDS reads and adds overlap
   uint32_t i = tid;
@@ -129,8 +131,8 @@ template <typename key_t> struct Cut {
 
 // key_at(i): order key of candidate i; index_at(i): its original index (only
 // read for candidates tied at T, and only when the tie group is cut).
-template <typename key_t, int KEY_BITS, typename KeyAt, typename IndexAt>
-__device__ __forceinline__ Cut<key_t> find_cut(Shared& sh, uint32_t k0, uint32_t k, int index_bits, KeyAt key_at,
+template <typename key_t, int KEY_BITS, typename KeyAt, typename IndexAt, typename Sh>
+__device__ __forceinline__ Cut<key_t> find_cut(Sh& sh, uint32_t k0, uint32_t k, int index_bits, KeyAt key_at,
                                       IndexAt index_at) {
   key_t prefix = 0, mask = 0;
   uint32_t need = k;
@@ -167,8 +169,8 @@ __device__ __forceinline__ Cut<key_t> find_cut(Shared& sh, uint32_t k0, uint32_t
 // its loads (coalesced, independent of the outcome) overlap; emit(i, o, what
 // fetch(i) returned) is called for every surviving candidate i with its output
 // slot o < k.
-template <typename Survives, typename Fetch, typename Emit>
-__device__ __forceinline__ void compact(Shared& sh, uint32_t k0, uint32_t k, Survives survives, Fetch fetch,
+template <typename Survives, typename Fetch, typename Emit, typename Sh>
+__device__ __forceinline__ void compact(Sh& sh, uint32_t k0, uint32_t k, Survives survives, Fetch fetch,
                                         Emit emit) {
   const uint32_t tid = threadIdx.x, nt = blockDim.x;
   const uint32_t waves = nt / kWave, wave = tid / kWave, lane = lane_id();
