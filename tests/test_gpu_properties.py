@@ -173,3 +173,19 @@ def test_recall_matches_closed_form(n, k, j, k_mult):
     recall = float(((v >= kth).sum(-1).double() / k).mean())
     expected = _closed_form_recall(k, k * k_mult // j, j)
     assert abs(recall - expected) < 0.02, (recall, expected)
+
+
+def test_row_longer_than_two_to_the_31():
+    """Positions beyond 2^31: index arithmetic must be 64-bit end to end."""
+    n = (1 << 31) + 4099
+    g = torch.Generator().manual_seed(31)
+    x = torch.randint(0, 255, (1, n), generator=g, dtype=torch.uint8)
+    x[0, -5:] = 255                      # the only 255s: winners at the very end of the row
+    xg = x.cuda()
+    for k, j, interleaved in [(64, 2, True), (1 << 16, 1, True), (96, 3, False)]:
+        v, i = _topk()(xg, k, -1, j=j, interleaved=interleaved)
+        ev, ei = oracle.topk(x, k, -1, j=j, interleaved=interleaved)
+        assert_same(v, i, ev, ei, f"k={k} j={j} interleaved={interleaved}")
+        assert int(i.max()) >= n - 5
+    del xg
+    torch.cuda.empty_cache()
