@@ -12,6 +12,10 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 constexpr int64_t kTargetWaves = 1024;
 // Sub-rows worth giving to one wave before a row is also cut into slabs.
 constexpr int64_t kSlabRun = 16;
+// Fewest sub-rows a wave scans when several share a tile: with runs of 2 the
+// hand-over costs more than the scan (measured at 16 sub-rows: 4 waves x 4 beat
+// 8 x 2 by 25-45 %).
+constexpr int64_t kMinRun = 4;
 // Buckets at least this long are folded when they do not fill a column tile;
 // below, merging the folded columns costs more than the idle lanes.
 constexpr int64_t kFoldMinLength = 128;
@@ -57,13 +61,13 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   // full/w pushes, plus (w-1)*j pushes to fold the other waves' queues.  Take
   // the largest w within 30 % of the cheapest (short-lived waves keep more of
   // the HBM bandwidth: measured, 8 waves x 4 sub-rows beats 4 x 8 at the
-  // headline shape), with every run at least j long and the LDS hand-over
-  // within its budget.
+  // headline shape), with every run at least max(j, 4) long and the LDS
+  // hand-over within its budget.
   const int cmp_size = es > 4 ? 8 : 4;
   int64_t cost[4] = {full, 0, 0, 0};
   int cands = 1;
   for (int cand = 2; cand <= 8; cand *= 2, ++cands) {
-    if (full / cand < j || merge_lds_bytes(pl.vec, j, cand, cmp_size) > kMergeLdsLimit) break;
+    if (full / cand < (j > kMinRun ? j : kMinRun) || merge_lds_bytes(pl.vec, j, cand, cmp_size) > kMergeLdsLimit) break;
     cost[cands] = full / cand + (int64_t)(cand - 1) * j;
   }
   int64_t best = cost[0];
