@@ -23,13 +23,14 @@ int check_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int
   return ATK_OK;
 }
 
-// Workspace of atk_topk: the stage-1 candidates, then stage 1's own scratch.
+// Workspace of atk_topk: the stage-1 candidates, then stage 1's own scratch,
+// then stage 2's.
 struct TopkPlan {
-  size_t cand_values_off, cand_indices_off, stage1_off, stage1_bytes, total;
+  size_t cand_values_off, cand_indices_off, stage1_off, stage1_bytes, select_off, select_bytes, total;
 };
 
 TopkPlan plan_topk(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype) {
-  TopkPlan p{0, 0, 0, 0, 0};
+  TopkPlan p{0, 0, 0, 0, 0, 0, 0};
   if (rows <= 0 || k0 <= 0) return p;
   p.stage1_bytes = atk_stage1_workspace_bytes(rows, n, k0, j, layout, dtype);
   if (k == k0) {
@@ -39,7 +40,9 @@ TopkPlan plan_topk(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int la
   const size_t vals = align_up((size_t)rows * (size_t)k0 * atk::elem_bytes(dtype), 256);
   p.cand_indices_off = vals;
   p.stage1_off = vals + align_up((size_t)rows * (size_t)k0 * sizeof(int64_t), 256);
-  p.total = p.stage1_off + p.stage1_bytes;
+  p.select_off = p.stage1_off + align_up(p.stage1_bytes, 256);
+  p.select_bytes = atk_select_workspace_bytes(rows, k0, k, dtype);
+  p.total = p.select_off + p.select_bytes;
   return p;
 }
 
@@ -57,6 +60,19 @@ int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64
   if (handled || rc2 != ATK_OK) return rc2;
   return atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout, dtype, values,
                                             indices, stream);
+}
+
+// Stage 2 over many workgroups per row when a row holds very many candidates,
+// else one workgroup per row.
+int run_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
+               int64_t index_bound, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+               hipStream_t stream) {
+  bool handled = false;
+  const int rc = atk::launch_multi_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
+                                          indices, ws, ws_bytes, stream, &handled);
+  if (handled || rc != ATK_OK) return rc;
+  return atk::launch_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values, indices,
+                            stream);
 }
 
 }  // namespace
@@ -93,18 +109,19 @@ int atk_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64
                     (hipStream_t)stream);
 }
 
-size_t atk_select_workspace_bytes(int64_t, int64_t, int64_t, int) { return 0; }
+size_t atk_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
+  return atk::multi_select_workspace_bytes(rows, k0, k, dtype);
+}
 
 int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
                int64_t k, int64_t index_bound, int dtype, void* values, int64_t* indices,
                void* ws, size_t ws_bytes, atk_stream_t stream) {
-  (void)ws; (void)ws_bytes;
   if (atk::elem_bytes(dtype) == 0) return ATK_ERR_DTYPE;
   if (rows < 0 || k0 < 0 || k < 0 || k > k0 || index_bound < 0) return ATK_ERR_K;
   if (rows == 0 || k == 0) return ATK_OK;
   if (!cand_values || !cand_indices || !values || !indices) return ATK_ERR_ARG;
-  return atk::launch_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype,
-                            values, indices, (hipStream_t)stream);
+  return run_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values, indices, ws,
+                    ws_bytes, (hipStream_t)stream);
 }
 
 size_t atk_topk_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int64_t k,
@@ -139,8 +156,8 @@ int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t
   const int64_t bound = (layout == ATK_CEIL_CHUNK || layout == ATK_INTERLEAVED_PADDED)
                             ? ((n + k0 - 1) / k0) * k0
                             : n;
-  return atk::launch_select(cand_values, cand_indices, rows, k0, k, bound, dtype, values,
-                            indices, (hipStream_t)stream);
+  return run_select(cand_values, cand_indices, rows, k0, k, bound, dtype, values, indices,
+                    base + p.select_off, p.select_bytes, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -38,4 +38,11 @@ int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t 
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
                   int64_t* indices, hipStream_t stream);
 
+// stage2_multi_select.hip: many workgroups per row, for rows with very many
+// candidates; needs a workspace.  `*handled` as above.
+size_t multi_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype);
+int launch_multi_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
+                        int64_t k, int64_t index_bound, int dtype, void* values, int64_t* indices, void* ws,
+                        size_t ws_bytes, hipStream_t stream, bool* handled);
+
 }  // namespace atk

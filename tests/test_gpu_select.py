@@ -1,0 +1,91 @@
+"""GPU parity of stage 2 alone (atk_select through the C ABI) against the CPU
+oracle: exact top-k of given candidates, ties to the lowest original index,
+survivors in candidate order.  Covers the one-workgroup kernel (keys in LDS and
+keys re-read from global memory) and the multi-workgroup chain of launches that
+takes rows with more than 65536 candidates."""
+import pytest
+import torch
+
+import oracle
+from helpers import assert_same
+
+pytestmark = pytest.mark.gpu
+
+
+def _select(cv, ci, k, bound):
+    from approx_topk import _native
+    v, i = _native.select(cv.cuda(), ci.cuda(), k, bound)
+    torch.cuda.synchronize()
+    return v, i
+
+
+def _candidates(rows, k0, dtype, seed, ties, bound):
+    g = torch.Generator().manual_seed(seed)
+    if ties:      # few distinct values: the cut falls inside a large group of equal keys
+        cv = torch.randint(-3, 4, (rows, k0), generator=g).to(dtype)
+    elif dtype.is_floating_point:
+        cv = torch.randn((rows, k0), generator=g).to(dtype)
+    else:
+        cv = torch.randint(-30000, 30000, (rows, k0), generator=g).to(dtype)
+    # distinct original indices below `bound`, in no particular order
+    ci = torch.stack([torch.randperm(bound, generator=g)[:k0] for _ in range(rows)]) if bound <= (1 << 22) else \
+        torch.stack([torch.randperm(k0, generator=g) * (bound // k0) + 1 for _ in range(rows)])
+    return cv, ci
+
+
+@pytest.mark.parametrize("rows,k0,k", [
+    (3, 1000, 100), (2, 40000, 777), (2, 70000, 30000),          # one workgroup per row
+    (2, 65537, 1), (3, 131072, 32768), (1, 300001, 150000), (2, 1 << 20, 1000), (5, 100000, 99999),
+])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.int64, torch.uint8])
+@pytest.mark.parametrize("ties", [False, True])
+def test_select_matches_oracle(rows, k0, k, dtype, ties):
+    if dtype == torch.uint8 and not ties:
+        pytest.skip("uint8 candidates are always tie-heavy")
+    bound = max(k0, 1 << 21)
+    cv, ci = _candidates(rows, k0, dtype, k0 + k, ties, bound)
+    if dtype == torch.uint8:
+        cv = cv.abs().to(dtype)
+    v, i = _select(cv, ci, k, bound)
+    ev, ei = oracle.stage2(cv, ci, k)
+    assert_same(v, i, ev, ei, f"rows={rows} k0={k0} k={k} {dtype} ties={ties}")
+
+
+def test_select_all_equal_and_wide_indices():
+    k0, k = 200000, 12345
+    bound = 1 << 40                      # four index digits of 11 bits
+    cv = torch.full((2, k0), 1.5)
+    cv[1, ::7] = float("nan")            # NaN ranks above everything, ties among NaN by index
+    g = torch.Generator().manual_seed(5)
+    ci = torch.stack([torch.randperm(k0, generator=g) * (bound // k0) + 3 for _ in range(2)])
+    v, i = _select(cv, ci, k, bound)
+    ev, ei = oracle.stage2(cv, ci, k)
+    assert_same(v, i, ev, ei, "all-equal rows")
+
+
+def test_select_under_graph_replay():
+    cv, ci = _candidates(2, 150000, torch.float32, 11, True, 1 << 21)
+    from approx_topk import _native
+    cvg, cig = cv.cuda(), ci.cuda()
+    _native.select(cvg, cig, 5000, 1 << 21)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        v, i = _native.select(cvg, cig, 5000, 1 << 21)
+    ev, ei = oracle.stage2(cv, ci, 5000)
+    for _ in range(3):
+        v.zero_(); i.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_same(v, i, ev, ei, "graph replay")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_topk_with_many_candidates(dtype, interleaved):
+    from approx_topk import topk
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn((2, 1 << 20), generator=g).to(dtype)
+    v, i = topk(x.cuda(), 32768, -1, j=2, k_mult=4, interleaved=interleaved)   # 131072 candidates per row
+    ev, ei = oracle.topk(x, 32768, -1, j=2, k_mult=4, interleaved=interleaved)
+    assert_same(v, i, ev, ei, f"{dtype} interleaved={interleaved}")
