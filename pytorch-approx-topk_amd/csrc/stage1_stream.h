@@ -804,14 +804,26 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
   word_t acc[N], in[N];
   ATK_STATIC_FOR(s, N) { acc[s] = M::empty(); in[s] = M::empty(); } ATK_STATIC_END;
   if (live) {
+    // four sources per round, their loads issued together
+    constexpr int kBatch = 4;
     const uint32_t sources = slabs * fold;
-    uint32_t slab = share / fold, f = share - slab * fold;
-    for (uint32_t src = share; src < sources; src += shares) {
-      const int64_t o = ((row * slabs + slab) * width + (int64_t)f * b + c) * J;
-      ATK_STATIC_FOR(s, J) { in[N - J + s] = M::make(part_values[o + s], part_pos[o + s] * fold + f); } ATK_STATIC_END;
-      merge_best<M, N>(acc, in);
-      f += shares;
-      while (f >= fold) { f -= fold; ++slab; }
+    for (uint32_t src0 = share; src0 < sources; src0 += shares * kBatch) {
+      typename E::raw_t got[kBatch][J];
+      uint32_t at[kBatch][J], which[kBatch];
+      ATK_STATIC_FOR(u, kBatch) {
+        const uint32_t src = src0 + u * shares;
+        const uint32_t clamped = src < sources ? src : share;  // a source that exists; ignored below
+        const uint32_t slab = clamped / fold, f = clamped - slab * fold;
+        which[u] = src < sources ? f : kEmptySlot;
+        const int64_t o = ((row * slabs + slab) * width + (int64_t)f * b + c) * J;
+        ATK_STATIC_FOR(s, J) { got[u][s] = part_values[o + s]; at[u][s] = part_pos[o + s]; } ATK_STATIC_END;
+      } ATK_STATIC_END;
+      ATK_STATIC_FOR(u, kBatch) {
+        if (which[u] != kEmptySlot) {
+          ATK_STATIC_FOR(s, J) { in[N - J + s] = M::make(got[u][s], at[u][s] * fold + which[u]); } ATK_STATIC_END;
+          merge_best<M, N>(acc, in);
+        }
+      } ATK_STATIC_END;
     }
   }
   for (uint32_t half = shares / 2; half >= 1; half /= 2) {

@@ -62,8 +62,11 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
                             : launch_w<E, J, 1>(pl, x, out, g, rows, stream);
   if (rc != ATK_OK || !pl.merge) return rc;
   const int64_t b = pl.width / pl.fold;  // buckets
-  uint32_t cb = kWave;                   // buckets per workgroup: a power of two, no more than needed
-  while (cb > 1 && (int64_t)(cb / 2) >= b) cb /= 2;
+  // buckets per workgroup: a power of two, no more than there are, and few
+  // enough that a thread folds at most about 32 of a bucket's partial queues
+  uint32_t cb = kWave;
+  const int64_t sources = (int64_t)pl.slabs * pl.fold;
+  while (cb > 1 && ((int64_t)(cb / 2) >= b || sources * cb > 32 * kMergeThreads)) cb /= 2;
   const int64_t blocks_per_row = (b + cb - 1) / cb;
   if (blocks_per_row * rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)),
