@@ -56,7 +56,7 @@ int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64
                                            indices, ws, ws_bytes, stream, &handled);
   if (handled || rc != ATK_OK) return rc;
   const int rc2 = atk::launch_stage1_contig(x, rows, n, row_stride, k0, j, layout, dtype, values, indices,
-                                            stream, &handled);
+                                            ws, ws_bytes, stream, &handled);
   if (handled || rc2 != ATK_OK) return rc2;
   return atk::launch_stage1_lane_per_bucket(x, rows, n, row_stride, k0, j, layout, dtype, values,
                                             indices, stream);
@@ -97,7 +97,9 @@ const char* atk_strerror(int status) {
 }
 
 size_t atk_stage1_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype) {
-  return atk::stage1_stream_workspace_bytes(rows, n, k0, j, layout, dtype);
+  const size_t a = atk::stage1_stream_workspace_bytes(rows, n, k0, j, layout, dtype);
+  const size_t c = atk::stage1_contig_workspace_bytes(rows, n, k0, j, layout, dtype);
+  return a > c ? a : c;
 }
 
 int atk_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,

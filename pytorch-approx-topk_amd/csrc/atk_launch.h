@@ -23,9 +23,10 @@ int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_str
                          size_t ws_bytes, hipStream_t stream, bool* handled);
 
 // stage1_contig_plan.hip: the contiguous layouts, through LDS.  `*handled` as above.
+size_t stage1_contig_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype);
 int launch_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                         int layout, int dtype, void* values, int64_t* indices, hipStream_t stream,
-                         bool* handled);
+                         int layout, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+                         hipStream_t stream, bool* handled);
 
 // fused_row_plan.hip: both stages in one kernel, one workgroup per row, for
 // batches of many rows whose candidates fit in LDS.  `*handled` as above.

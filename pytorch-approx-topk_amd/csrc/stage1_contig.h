@@ -12,7 +12,10 @@
 // 256 pieces takes a workgroup of its own, which goes through it in chunks of
 // 256 pieces; a thread's queue then lives across the chunks (its pieces come
 // in increasing position, so a newcomer still only displaces what it beats
-// strictly).
+// strictly).  When that leaves too few workgroups for the GPU (few rows of few,
+// very long buckets), a bucket's chunks are shared out over `slabs` workgroups,
+// which park their J best as merge words in a workspace, and
+// `contig_merge_kernel` (one wave per bucket) combines them.
 //
 // LDS placement.  Element i of the span sits at i + i/32 words' worth of
 // elements (one 4-byte word of padding per 32 elements): the 4-byte writes of a
@@ -53,6 +56,8 @@ struct Geom {
   uint32_t sure;         // the shortest piece of any thread (one chunk; chunks but the last are full)
   uint32_t chunks;       // > 1: one bucket per workgroup, scanned in that many chunks
   uint32_t groups;       // workgroups per row
+  uint32_t slabs;        // > 1 (only with chunks > 1): workgroups sharing a bucket's chunks
+  uint32_t slab_chunks;  // chunks per slab; the last slab also takes the remainder
 };
 
 // How a thread's queue holds values: in compare form (fast; no NaN may be
@@ -79,8 +84,8 @@ template <typename E> __device__ __forceinline__ uint32_t lds_slot(uint32_t i) {
 template <typename E, int J, int V, typename F>
 __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict__ xr,
                                              typename E::raw_t* __restrict__ values,
-                                             int64_t* __restrict__ indices, int64_t row, uint32_t group,
-                                             const Geom& g, unsigned char* lds) {
+                                             int64_t* __restrict__ indices, void* __restrict__ partial,
+                                             int64_t row, uint32_t group, const Geom& g, unsigned char* lds) {
   using raw_t = typename E::raw_t;
   using T = typename F::T;
   using M = typename F::M;
@@ -93,7 +98,11 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
   const uint32_t t = threadIdx.x;
   const uint32_t pieces = 1u << g.pieces_log2;
   const uint32_t per_group = kThreads >> g.pieces_log2;  // buckets per workgroup
-  const uint32_t c0 = group * per_group;
+  const uint32_t slab = g.slabs > 1 ? group % g.slabs : 0u;
+  const uint32_t c0 = g.slabs > 1 ? group / g.slabs : group * per_group;
+  // the chunks of this workgroup
+  const uint32_t it0 = slab * g.slab_chunks;
+  const uint32_t it1 = (g.slabs == 1 || slab + 1 == g.slabs) ? g.chunks : it0 + g.slab_chunks;
   const uint32_t c = c0 + (t >> g.pieces_log2);
   const uint32_t piece = t & (pieces - 1);
   const bool has = c < g.b;
@@ -104,7 +113,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
 
   T q[J];
   uint32_t pos[J];
-  for (uint32_t it = 0; it < g.chunks; ++it) {
+  for (uint32_t it = it0; it < it1; ++it) {
     // the span this round: all the workgroup's buckets, or one chunk of its only bucket
     uint32_t e0, e1;
     if (g.chunks == 1) {
@@ -116,7 +125,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
       e1 = e0 + kChunk < end ? e0 + kChunk : end;
     }
     const uint32_t a0 = e0 & ~(uint32_t)(V - 1);  // packs are aligned in the row
-    if (it != 0) __syncthreads();                 // the last round's reads are done
+    if (it != it0) __syncthreads();               // the last round's reads are done
 
     bool nan = false;
     const uint32_t packs = (e1 - a0 + V - 1) / V;
@@ -180,7 +189,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
       const uint32_t first = start + lo;  // position in the row
       const uint32_t li = first - a0;     // position in the span
       uint32_t s = 0;
-      if (it == 0) {  // every piece of the first round holds at least J elements
+      if (it == it0) {  // every piece of a workgroup's first round holds at least J elements
         ATK_STATIC_FOR(u, J) {
           stream::push<T, J, u>(q, pos, F::conv(data[lds_slot<E>(li + u)]), first + u);
         } ATK_STATIC_END;
@@ -221,12 +230,17 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
     }
   }
   if (has && piece == 0) {
-    const int64_t o = (row * g.b + c) * J;
-    ATK_STATIC_FOR(sl, J) {
-      const uint32_t p = M::pos(acc[N - J + sl]);
-      values[o + sl] = (int64_t)p < g.n ? xr[p] : E::pad_raw;
-      indices[o + sl] = p;
-    } ATK_STATIC_END;
+    if (g.slabs > 1) {
+      word_t* park = reinterpret_cast<word_t*>(partial) + ((row * g.b + c) * g.slabs + slab) * N;
+      ATK_STATIC_FOR(sl, N) { park[sl] = acc[sl]; } ATK_STATIC_END;
+    } else {
+      const int64_t o = (row * g.b + c) * J;
+      ATK_STATIC_FOR(sl, J) {
+        const uint32_t p = M::pos(acc[N - J + sl]);
+        values[o + sl] = (int64_t)p < g.n ? xr[p] : E::pad_raw;
+        indices[o + sl] = p;
+      } ATK_STATIC_END;
+    }
   }
   return true;
 }
@@ -236,17 +250,53 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
 template <typename E, int J, int V>
 __global__ __launch_bounds__(kThreads) void contig_kernel(const typename E::raw_t* __restrict__ x,
                                                           typename E::raw_t* __restrict__ values,
-                                                          int64_t* __restrict__ indices, const Geom g) {
+                                                          int64_t* __restrict__ indices,
+                                                          void* __restrict__ partial, const Geom g) {
   extern __shared__ __align__(16) unsigned char contig_lds[];
   const uint32_t row32 = blockIdx.x / g.groups;
   const uint32_t group = blockIdx.x - row32 * g.groups;
   const int64_t row = row32;
   const typename E::raw_t* xr = x + row * g.row_stride;
-  if (scan_buckets<E, J, V, CmpForm<E>>(xr, values, indices, row, group, g, contig_lds)) return;
+  if (scan_buckets<E, J, V, CmpForm<E>>(xr, values, indices, partial, row, group, g, contig_lds)) return;
   if constexpr (Cmp<E>::has_nan) {
     __syncthreads();
-    scan_buckets<E, J, V, KeyForm<E>>(xr, values, indices, row, group, g, contig_lds);
+    scan_buckets<E, J, V, KeyForm<E>>(xr, values, indices, partial, row, group, g, contig_lds);
   }
+}
+
+// Combines the `slabs` partial results of every bucket: one wave per bucket,
+// lane l folding slabs l, l + 64, ..., then pairwise by lane shuffles.
+template <typename E, int J>
+__global__ __launch_bounds__(64) void contig_merge_kernel(const typename E::raw_t* __restrict__ x,
+                                                         const void* __restrict__ partial,
+                                                         typename E::raw_t* __restrict__ values,
+                                                         int64_t* __restrict__ indices, const Geom g) {
+  using M = MergeWord<E>;
+  using word_t = typename M::word_t;
+  constexpr int N = J == 3 ? 4 : J;
+  const int64_t bucket = blockIdx.x;  // row * b + c
+  const int64_t row = bucket / g.b;
+  const uint32_t c = (uint32_t)(bucket - row * g.b);
+  const uint32_t lane = threadIdx.x;
+  const word_t* lists = reinterpret_cast<const word_t*>(partial) + bucket * g.slabs * N;
+  word_t acc[N], in[N];
+  ATK_STATIC_FOR(sl, N) { acc[sl] = M::empty(); } ATK_STATIC_END;
+  for (uint32_t s = lane; s < g.slabs; s += 64) {
+    ATK_STATIC_FOR(sl, N) { in[sl] = lists[(int64_t)s * N + sl]; } ATK_STATIC_END;
+    stream::merge_best<M, N>(acc, in);
+  }
+  for (int half = 32; half >= 1; half /= 2) {
+    ATK_STATIC_FOR(sl, N) { in[sl] = M::from_lane(acc[sl], (int)lane + half); } ATK_STATIC_END;
+    stream::merge_best<M, N>(acc, in);  // meaningful in the lanes below `half`, which are the ones read next
+  }
+  if (lane != 0) return;
+  const typename E::raw_t* xr = x + row * g.row_stride;
+  const int64_t o = (row * g.b + c) * J;
+  ATK_STATIC_FOR(sl, J) {
+    const uint32_t p = M::pos(acc[N - J + sl]);
+    values[o + sl] = (int64_t)p < g.n ? xr[p] : E::pad_raw;
+    indices[o + sl] = p;
+  } ATK_STATIC_END;
 }
 
 // ---------------------------------------------------------------------------
@@ -257,6 +307,7 @@ struct Plan {
   int vec;           // V
   Geom geom;         // row_stride is filled in at launch
   size_t lds_bytes;  // dynamic LDS per workgroup
+  size_t ws_bytes;   // workspace for the slabs' partial results
 };
 
 // `aligned`: base pointer and row stride allow 16-byte loads.
@@ -264,7 +315,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
-                 int64_t* indices, hipStream_t stream);
+                 int64_t* indices, void* ws, hipStream_t stream);
 
 }  // namespace contig
 }  // namespace atk

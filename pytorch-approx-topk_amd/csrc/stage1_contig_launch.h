@@ -9,42 +9,45 @@ namespace contig {
 
 template <typename E, int J, int V>
 static int launch_one(const Plan& pl, const Geom& g, const typename E::raw_t* x, int64_t rows,
-                      typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+                      typename E::raw_t* values, int64_t* indices, void* ws, hipStream_t stream) {
   const int64_t groups = rows * (int64_t)g.groups;
   if (groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   hipLaunchKernelGGL((contig_kernel<E, J, V>), dim3((unsigned)groups), dim3(kThreads), pl.lds_bytes, stream, x,
-                     values, indices, g);
+                     values, indices, ws, g);
+  if (g.slabs > 1)
+    hipLaunchKernelGGL((contig_merge_kernel<E, J>), dim3((unsigned)(rows * g.b)), dim3(64), 0, stream, x,
+                       (const void*)ws, values, indices, g);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
 template <typename E, int J>
 static int launch_j(const Plan& pl, const Geom& g, const typename E::raw_t* x, int64_t rows,
-                    typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+                    typename E::raw_t* values, int64_t* indices, void* ws, hipStream_t stream) {
   constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
-  return pl.vec > 1 ? launch_one<E, J, VF>(pl, g, x, rows, values, indices, stream)
-                    : launch_one<E, J, 1>(pl, g, x, rows, values, indices, stream);
+  return pl.vec > 1 ? launch_one<E, J, VF>(pl, g, x, rows, values, indices, ws, stream)
+                    : launch_one<E, J, 1>(pl, g, x, rows, values, indices, ws, stream);
 }
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
-                 int64_t* indices, hipStream_t stream) {
+                 int64_t* indices, void* ws, hipStream_t stream) {
   using raw_t = typename E::raw_t;
   Geom g = pl.geom;
   g.row_stride = row_stride;
   const raw_t* xs = static_cast<const raw_t*>(x);
   raw_t* vs = static_cast<raw_t*>(values);
   switch (j) {
-    case 1: return launch_j<E, 1>(pl, g, xs, rows, vs, indices, stream);
-    case 2: return launch_j<E, 2>(pl, g, xs, rows, vs, indices, stream);
-    case 3: return launch_j<E, 3>(pl, g, xs, rows, vs, indices, stream);
-    case 4: return launch_j<E, 4>(pl, g, xs, rows, vs, indices, stream);
+    case 1: return launch_j<E, 1>(pl, g, xs, rows, vs, indices, ws, stream);
+    case 2: return launch_j<E, 2>(pl, g, xs, rows, vs, indices, ws, stream);
+    case 3: return launch_j<E, 3>(pl, g, xs, rows, vs, indices, ws, stream);
+    case 4: return launch_j<E, 4>(pl, g, xs, rows, vs, indices, ws, stream);
   }
   return ATK_ERR_J;
 }
 
 #define ATK_INSTANTIATE_CONTIG(DT)                                                                \
   template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int, void*, \
-                                      int64_t*, hipStream_t);
+                                      int64_t*, void*, hipStream_t);
 
 }  // namespace contig
 }  // namespace atk

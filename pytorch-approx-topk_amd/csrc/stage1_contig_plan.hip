@@ -4,6 +4,11 @@
 namespace atk {
 namespace contig {
 
+namespace {
+// Workgroups wanted in the grid before long buckets are left whole.
+constexpr int64_t kTargetGroups = 1024;
+}  // namespace
+
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned) {
   Plan pl{};
   pl.ok = false;
@@ -38,6 +43,20 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   }
   const int64_t per_group = kThreads >> lg;
   g.groups = (uint32_t)((b + per_group - 1) / per_group);
+  // Few rows of few very long buckets: share a bucket's chunks out over
+  // workgroups (at least two chunks each, so that every workgroup starts on a
+  // full chunk) until the grid has about kTargetGroups of them.
+  g.slabs = 1;
+  g.slab_chunks = g.chunks;
+  if (g.chunks >= 4 && rows * b < kTargetGroups / 2) {
+    int64_t slabs = (kTargetGroups + rows * b - 1) / (rows * b);
+    if (slabs > g.chunks / 2) slabs = g.chunks / 2;
+    if (slabs > 256) slabs = 256;
+    g.slabs = (uint32_t)slabs;
+    g.slab_chunks = g.chunks / g.slabs;
+    g.groups = (uint32_t)(b * slabs);
+    pl.ws_bytes = (size_t)rows * (size_t)b * (size_t)slabs * 4 * (es == 8 ? 16 : 8);
+  }
   if (rows * (int64_t)g.groups > 0x7fffffffll) return pl;
 
   pl.vec = aligned ? stream::full_vec(es) : 1;
@@ -53,18 +72,28 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
 
 }  // namespace contig
 
+size_t stage1_contig_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype) {
+  const contig::Plan a = contig::make_plan(rows, n, k0, j, layout, dtype, true);
+  const contig::Plan u = contig::make_plan(rows, n, k0, j, layout, dtype, false);
+  size_t need = 0;
+  if (a.ok && a.ws_bytes > need) need = a.ws_bytes;
+  if (u.ok && u.ws_bytes > need) need = u.ws_bytes;
+  return need;
+}
+
 int launch_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                         int layout, int dtype, void* values, int64_t* indices, hipStream_t stream,
-                         bool* handled) {
+                         int layout, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+                         hipStream_t stream, bool* handled) {
   const int es = elem_bytes(dtype);
   const int vf = es ? stream::full_vec(es) : 1;
   const bool aligned = ((uintptr_t)x % 16 == 0) && (row_stride % vf == 0);
   const contig::Plan pl = contig::make_plan(rows, n, k0, j, layout, dtype, aligned);
   *handled = pl.ok;
   if (!pl.ok) return ATK_OK;
+  if (pl.ws_bytes && (!ws || ws_bytes < pl.ws_bytes || (uintptr_t)ws % 16 != 0)) return ATK_ERR_WORKSPACE;
   int rc = ATK_ERR_DTYPE;
   ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
-                   rc = contig::launch_typed<E>(pl, x, rows, row_stride, j, values, indices, stream));
+                   rc = contig::launch_typed<E>(pl, x, rows, row_stride, j, values, indices, ws, stream));
   return rc;
 }
 

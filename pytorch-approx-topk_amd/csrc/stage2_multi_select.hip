@@ -297,15 +297,16 @@ struct MultiPlan {
 
 // The multi-workgroup select is taken when it is expected to be the faster one.
 // Measured on an MI355X (fp32 and fp16, k = k0/4): the chain of launches costs
-// about 50 us plus 11.5 us per million candidates of the whole batch; one
-// workgroup per row costs about 1 us per thousand candidates of a row, rows
-// running side by side up to about 96 of them.  Rows of up to 48K candidates
+// about 45 us plus 11.7 us per million candidates of the whole batch; one
+// workgroup per row is bound by what one CU can read, about 1.2 us per thousand
+// candidates of a row (rows run side by side), until the batch as a whole is
+// bound by HBM, which the chain is as well.  Rows of up to 48K candidates
 // always stay with one workgroup (its keys then sit in LDS).
 constexpr int64_t kMultiMinCandidates = 49152;
 
 bool multi_is_faster(int64_t rows, int64_t k0) {
-  const double multi = 50.0 + 11.5e-6 * (double)rows * (double)k0;
-  const double single = 1e-3 * (double)k0 * (rows > 96 ? (double)rows / 96.0 : 1.0);
+  const double multi = 45.0 + 11.7e-6 * (double)rows * (double)k0;
+  const double single = 1.2e-3 * (double)k0;
   return multi < single;
 }
 
