@@ -78,13 +78,17 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   pl.waves = w;
 
   // Slabs: only when the grid would still be small and the runs are long.
+  // Once a row is cut at all (the merge launch is then paid for anyway), short
+  // queues (j <= 2, whose merge is cheap) are cut for twice as many waves:
+  // measured 41 -> 28 us on fp32 [2, 2^24] with 4096 buckets, 57 -> 52 us on
+  // [1, 2^26] with 16384 buckets at j = 2; j = 4 loses a little.
   pl.slabs = 1;
   const int64_t waves = rows * pl.col_tiles * w;
-  if (waves < kTargetWaves) {
-    int64_t slabs = (kTargetWaves + waves - 1) / waves;
-    const int64_t most = full / (w * kSlabRun);
+  const int64_t most = full / (w * kSlabRun);
+  if (waves < kTargetWaves && most > 1) {
+    const int64_t target = j <= 2 ? 2 * kTargetWaves : kTargetWaves;
+    int64_t slabs = (target + waves - 1) / waves;
     if (slabs > most) slabs = most;
-    if (slabs < 1) slabs = 1;
     pl.slabs = (uint32_t)slabs;
   }
   pl.slab_len = (uint32_t)(full / pl.slabs);
