@@ -29,8 +29,12 @@ using stream::kWave;
 
 // pos_t: uint16_t when every sub-row number fits, else uint32_t.  PACKED: packed
 // 16-bit queues (stage1_stream.h).
+// The SGPR cap keeps eight waves per SIMD possible (beyond 96 scalar registers
+// only seven fit, whatever the vector registers allow): for 1024 fp16 rows of
+// 32768 with 8192 candidates that is a fourth workgroup per CU and every row
+// resident at once.
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
-__global__ __launch_bounds__(kWave * MAXW) void fused_row_kernel(
+__global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) void fused_row_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
     int64_t* __restrict__ indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t hand_off,
     uint32_t k0, uint32_t k, int index_bits) {
