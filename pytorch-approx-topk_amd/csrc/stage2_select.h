@@ -25,6 +25,9 @@ constexpr int kMaxWaves = 16;
 // key is nearly constant among top-k candidates -- do not serialise on one LDS
 // address; the odd stride spreads equal digits of different copies over banks.
 constexpr int kCopyStride = 257;
+// Tie groups up to this size are cut by ranking their listed indices in one
+// wave instead of by radix passes over all candidates.
+constexpr int kTieList = 64;
 
 template <int COPIES> struct SharedT {
   static constexpr int kCopies = COPIES;
@@ -34,6 +37,10 @@ template <int COPIES> struct SharedT {
   uint32_t digit;
   uint32_t need;
   uint32_t bin_count;
+  // a short tie group, listed: original indices of the candidates with key == T
+  uint32_t tie_count;
+  uint64_t tie_index[kTieList];
+  uint64_t index_cut;
 };
 using Shared = SharedT<8>;  // the stand-alone select kernel; the fused kernel takes fewer copies to save LDS
 
@@ -147,7 +154,25 @@ __device__ __forceinline__ Cut<key_t> find_cut(Sh& sh, uint32_t k0, uint32_t k, 
   }
   Cut<key_t> cut{prefix, ~0ull};
   const uint32_t ties = sh.bin_count;  // candidates with key == T
-  if (need < ties) {                   // uniform over the workgroup
+  if (need < ties && ties <= (uint32_t)kTieList) {  // uniform over the workgroup
+    // list the tied candidates' indices (in any order), then one wave finds
+    // the need-th smallest by counting, for every index, the smaller ones
+    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    if (tid == 0) sh.tie_count = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < k0; i += nt) {
+      if (key_at(i) == cut.T) sh.tie_index[atomicAdd(&sh.tie_count, 1u)] = index_at(i);
+    }
+    __syncthreads();
+    if (tid < (uint32_t)kWave) {
+      const uint64_t mine = tid < ties ? sh.tie_index[tid] : ~0ull;
+      uint32_t smaller = 0;
+      for (uint32_t m = 0; m < ties; ++m) smaller += sh.tie_index[m] < mine ? 1u : 0u;
+      if (tid < ties && smaller == need - 1) sh.index_cut = mine;
+    }
+    __syncthreads();
+    cut.index_cut = sh.index_cut;
+  } else if (need < ties) {
     uint64_t iprefix = 0, imask = 0;
     for (int shift = ((index_bits + 7) / 8 - 1) * 8; shift >= 0; shift -= 8) {
       radix_pass<false>(sh, k0, need, [&](uint32_t i) -> int {
