@@ -2,7 +2,7 @@
 oracle: exact top-k of given candidates, ties to the lowest original index,
 survivors in candidate order.  Covers the one-workgroup kernel (keys in LDS and
 keys re-read from global memory) and the multi-workgroup chain of launches that
-takes rows with more than 65536 candidates."""
+takes rows with very many candidates."""
 import pytest
 import torch
 
@@ -34,7 +34,8 @@ def _candidates(rows, k0, dtype, seed, ties, bound):
 
 
 @pytest.mark.parametrize("rows,k0,k", [
-    (3, 1000, 100), (2, 40000, 777), (2, 70000, 30000),          # one workgroup per row
+    (5, 64, 10), (300, 512, 64), (7, 1024, 1000), (3, 100, 100), (9, 65, 1), (130, 300, 299),
+    (3, 1025, 100), (2, 40000, 777), (2, 70000, 30000),          # one workgroup per row
     (2, 65537, 1), (3, 131072, 32768), (1, 300001, 150000), (2, 1 << 20, 1000), (5, 100000, 99999),
 ])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.int64, torch.uint8])
