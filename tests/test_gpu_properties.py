@@ -125,26 +125,33 @@ def test_random_shapes_against_oracle():
 
 def test_hip_graph_replay_matches_eager():
     topk = _topk()
-    x = torch.randn(64, 1 << 16, device="cuda")
-    y = torch.randn(256, 8192, device="cuda", dtype=torch.float16)
+    # (input, k, kwargs): streaming kernel; fused kernel; few long buckets (folded, slabs + merge);
+    # contiguous buckets; two kernels with a select that keeps > 48 KiB of keys in LDS; the
+    # multi-workgroup select chain
+    cases = [
+        (torch.randn(64, 1 << 16, device="cuda"), 4096, dict(j=2)),
+        (torch.randn(256, 8192, device="cuda", dtype=torch.float16), 256, dict(j=4, k_mult=4)),
+        (torch.randn(8, 1 << 18, device="cuda"), 64, dict(j=2)),
+        (torch.randn(16, 1 << 16, device="cuda"), 1024, dict(j=2, interleaved=False)),
+        (torch.randn(2, 1 << 20, device="cuda"), 8192, dict(j=2, k_mult=2)),
+        (torch.randn(1, 1 << 20, device="cuda"), 32768, dict(j=1, k_mult=4)),
+    ]
     for _ in range(2):   # warm up allocator and library state outside the capture
-        topk(x, 4096, -1, j=2)
-        topk(y, 256, -1, j=4, k_mult=4)
+        for x, k, kw in cases:
+            topk(x, k, -1, **kw)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        out_a = topk(x, 4096, -1, j=2)
-        out_b = topk(y, 256, -1, j=4, k_mult=4)
+        outs = [topk(x, k, -1, **kw) for x, k, kw in cases]
     for rep in range(4):
-        x.normal_()
-        y.normal_()
-        ea = topk(x, 4096, -1, j=2)          # eager work between replays
-        eb = topk(y, 256, -1, j=4, k_mult=4)
+        for x, _, _ in cases:
+            x.normal_()
+        eager = [topk(x, k, -1, **kw) for x, k, kw in cases]   # eager work between replays
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(out_a[0], ea[0]) and torch.equal(out_a[1], ea[1]), f"replay {rep}"
-        assert torch.equal(out_b[0], eb[0]) and torch.equal(out_b[1], eb[1]), f"replay {rep}"
+        for n, (got, want) in enumerate(zip(outs, eager)):
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), f"replay {rep}, case {n}"
 
 
 def test_side_stream():
