@@ -407,3 +407,24 @@ def test_contiguous_buckets_unaligned_rows():
     v, i = _topk()(wide.cuda()[:, 3:30003], 20, -1, j=2, interleaved=False)
     ev, ei = oracle_topk(wide[:, 3:30003].contiguous(), 20, -1, j=2, interleaved=False)
     assert_same(v, i, ev, ei, "misaligned view")
+
+
+# ---- gradient: values are a gather of the input, so their gradient scatters back ----
+
+@pytest.mark.parametrize("k,j,k_mult,dim,interleaved", [(64, 2, 1, -1, True), (32, 4, 4, -1, True), (16, 1, 2, -1, False),
+                                                      (4, 4, 1, 0, True)])
+def test_gradient_scatters_to_the_selected_positions(k, j, k_mult, dim, interleaved):
+    from approx_topk.experimental.differentiable import topk as topk_with_gradient
+    x = cpu_randn((6, 512), 3).cuda().requires_grad_(True)
+    v, i = topk_with_gradient(x, k, dim, j=j, k_mult=k_mult, interleaved=interleaved)
+    pv, pi = _topk()(x.detach(), k, dim, j=j, k_mult=k_mult, interleaved=interleaved)
+    assert torch.equal(v.detach(), pv) and torch.equal(i, pi) and not i.requires_grad
+    w = torch.randn_like(v)
+    (v * w).sum().backward()
+    expect = torch.zeros_like(x).scatter(dim, i, w)
+    assert torch.equal(x.grad, expect)
+    # the same through plain torch ops on the returned indices
+    x2 = x.detach().clone().requires_grad_(True)
+    (x2.gather(dim, i) * w).sum().backward()
+    assert torch.equal(x.grad, x2.grad)
+

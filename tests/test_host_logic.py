@@ -119,3 +119,4 @@ def test_rows_view():
     assert t.is_contiguous() and (rows, n, step) == (9, 10, 10)
     t, rows, n, step = _native.rows_view(x.movedim(1, -1))
     assert t.is_contiguous() and (rows, n, step) == (30, 4, 4)
+
