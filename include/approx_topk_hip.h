@@ -118,6 +118,23 @@ int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride,
              void* values, int64_t* indices,
              void* ws, size_t ws_bytes, atk_stream_t stream);
 
+/*
+ * The same two entry points with int32 indices, for consumers that gather with
+ * 32-bit offsets (the index write is two thirds of the output traffic of
+ * atk_stage1 on 4-byte elements).  No counterpart in the reference, whose
+ * outputs are int64 (priority_queue.py:67).  Workspace as for the int64
+ * versions.  ATK_ERR_TOO_LARGE when a row (its padded length, for the padded
+ * layouts) has positions beyond 2^31 - 1.
+ */
+int atk_stage1_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride,
+                   int64_t k0, int j, int layout, int dtype,
+                   void* values, int32_t* indices,
+                   void* ws, size_t ws_bytes, atk_stream_t stream);
+int atk_topk_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride,
+                 int64_t k0, int j, int64_t k, int layout, int dtype,
+                 void* values, int32_t* indices,
+                 void* ws, size_t ws_bytes, atk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

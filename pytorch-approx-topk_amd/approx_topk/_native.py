@@ -30,6 +30,9 @@ _SIGNATURES = {
     "atk_stage1": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4 + [ctypes.c_int] * 3
                    + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
                       ctypes.c_void_p]),
+    "atk_stage1_i32": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4 + [ctypes.c_int] * 3
+                       + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                          ctypes.c_void_p]),
     "atk_select_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 3 + [ctypes.c_int]),
     "atk_select": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int64] * 4
                    + [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
@@ -40,6 +43,10 @@ _SIGNATURES = {
                                                                            ctypes.c_int, ctypes.c_int]
                  + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
                     ctypes.c_void_p]),
+    "atk_topk_i32": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4 + [ctypes.c_int, ctypes.c_int64,
+                                                                               ctypes.c_int, ctypes.c_int]
+                     + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                        ctypes.c_void_p]),
 }
 
 
@@ -126,19 +133,23 @@ def rows_view(xs: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
     return xs, rows, n, step
 
 
-def stage1(xs: torch.Tensor, k0: int, j: int, layout: int) -> tuple[torch.Tensor, torch.Tensor]:
-    """Per-bucket top-j along the last dim: (values[..., k0], indices[..., k0])."""
+def stage1(xs: torch.Tensor, k0: int, j: int, layout: int,
+           index_dtype: torch.dtype = torch.int64) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-bucket top-j along the last dim: (values[..., k0], indices[..., k0]).
+
+    ``index_dtype``: torch.int64 (the operator's contract) or torch.int32."""
     require_gpu(xs)
     L = lib()
     xs, rows, n, step = rows_view(xs)
     code = dtype_code(xs.dtype)
     shape = list(xs.shape[:-1]) + [k0]
     values = torch.empty(shape, dtype=xs.dtype, device=xs.device)
-    indices = torch.empty(shape, dtype=torch.int64, device=xs.device)
+    indices = torch.empty(shape, dtype=index_dtype, device=xs.device)
+    entry = L.atk_stage1 if index_dtype == torch.int64 else L.atk_stage1_i32
     with _on_device(xs.device):
         need = L.atk_stage1_workspace_bytes(rows, n, k0, j, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
-        check(L.atk_stage1(xs.data_ptr(), rows, n, step, k0, j, layout, code,
+        check(entry(xs.data_ptr(), rows, n, step, k0, j, layout, code,
                            values.data_ptr(), indices.data_ptr(),
                            ws.data_ptr() if ws is not None else None, need, _stream(xs.device)))
     return values, indices
@@ -165,7 +176,8 @@ def select(cand_values: torch.Tensor, cand_indices: torch.Tensor, k: int,
     return values, indices
 
 
-def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int) -> tuple[torch.Tensor, torch.Tensor]:
+def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int,
+         index_dtype: torch.dtype = torch.int64) -> tuple[torch.Tensor, torch.Tensor]:
     """Stage 1 (k0 candidates) and stage 2 (k survivors) along the last dim."""
     require_gpu(xs)
     L = lib()
@@ -173,11 +185,12 @@ def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int) -> tuple[torch.
     code = dtype_code(xs.dtype)
     shape = list(xs.shape[:-1]) + [k]
     values = torch.empty(shape, dtype=xs.dtype, device=xs.device)
-    indices = torch.empty(shape, dtype=torch.int64, device=xs.device)
+    indices = torch.empty(shape, dtype=index_dtype, device=xs.device)
+    entry = L.atk_topk if index_dtype == torch.int64 else L.atk_topk_i32
     with _on_device(xs.device):
         need = L.atk_topk_workspace_bytes(rows, n, k0, j, k, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
-        check(L.atk_topk(xs.data_ptr(), rows, n, step, k0, j, k, layout, code,
+        check(entry(xs.data_ptr(), rows, n, step, k0, j, k, layout, code,
                          values.data_ptr(), indices.data_ptr(),
                          ws.data_ptr() if ws is not None else None, need, _stream(xs.device)))
     return values, indices

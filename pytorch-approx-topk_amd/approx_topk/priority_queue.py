@@ -46,6 +46,7 @@ def _topk(
     k_mult: int = 1,
     interleaved: bool = True,
     multithread_buckets: bool | None = False,
+    index_dtype: torch.dtype = torch.int64,
 ) -> tuple[Tensor, Tensor]:
     """Approximate top-``k`` of ``xs`` along ``dim``.
 
@@ -75,7 +76,8 @@ def _topk(
     k0 = k * k_mult
 
     if k0 == 0:
-        return _empty_result(xs, 0, dim)
+        values, indices = _empty_result(xs, 0, dim)
+        return values, indices.to(index_dtype)
     if j < 1 or j > 4:
         raise RuntimeError("topk: j must 0 < j < 5")
     if k0 % j != 0:
@@ -85,7 +87,8 @@ def _topk(
         raise RuntimeError("topk: k must not be larger than topk size")
     _native.require_gpu(xs)
     if xs.numel() == 0:
-        return _empty_result(xs, k, dim)
+        values, indices = _empty_result(xs, k, dim)
+        return values, indices.to(index_dtype)
 
     layout = _native.INTERLEAVED if interleaved else _native.BALANCED
     rows = xs if xs.ndim else xs.reshape(1)
@@ -93,9 +96,9 @@ def _topk(
     if moved:
         rows = rows.movedim(dim, -1)
     if k_mult == 1:
-        values, indices = _native.stage1(rows, k0, j, layout)
+        values, indices = _native.stage1(rows, k0, j, layout, index_dtype)
     else:
-        values, indices = _native.topk(rows, k0, j, k, layout)
+        values, indices = _native.topk(rows, k0, j, k, layout, index_dtype)
     if moved:
         values = values.movedim(-1, dim).contiguous()
         indices = indices.movedim(-1, dim).contiguous()

@@ -49,7 +49,7 @@ TopkPlan plan_topk(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int la
 // Stage 1 through the streaming kernels when they take the shape, else the
 // general kernel.
 int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-               int layout, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+               int layout, int dtype, void* values, atk::IndexOut indices, void* ws, size_t ws_bytes,
                hipStream_t stream) {
   bool handled = false;
   const int rc = atk::launch_stage1_stream(x, rows, n, row_stride, k0, j, layout, dtype, values,
@@ -65,7 +65,7 @@ int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64
 // Stage 2 over many workgroups per row when a row holds very many candidates,
 // else one workgroup per row.
 int run_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
-               int64_t index_bound, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+               int64_t index_bound, int dtype, void* values, atk::IndexOut indices, void* ws, size_t ws_bytes,
                hipStream_t stream) {
   bool handled = false;
   const int rc = atk::launch_multi_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
@@ -73,6 +73,51 @@ int run_select(const void* cand_values, const int64_t* cand_indices, int64_t row
   if (handled || rc != ATK_OK) return rc;
   return atk::launch_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values, indices,
                             stream);
+}
+
+// Positions a layout can report: the row, or the padded row of the arg-max layouts.
+int64_t index_bound_of(int64_t n, int64_t k0, int layout) {
+  return (layout == ATK_CEIL_CHUNK || layout == ATK_INTERLEAVED_PADDED) ? ((n + k0 - 1) / k0) * k0 : n;
+}
+
+// int32 indices must be able to hold every position.
+bool fits_narrow(int64_t n, int64_t k0, int layout) { return index_bound_of(n, k0, layout) <= 0x7fffffffll; }
+
+int do_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int layout,
+              int dtype, void* values, atk::IndexOut indices, void* ws, size_t ws_bytes, hipStream_t stream) {
+  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices.base);
+  if (rc != ATK_OK || k0 == 0 || rows == 0) return rc;
+  if (indices.narrow && !fits_narrow(n, k0, layout)) return ATK_ERR_TOO_LARGE;
+  const size_t need = atk_stage1_workspace_bytes(rows, n, k0, j, layout, dtype);
+  if (need && (!ws || ws_bytes < need)) return ATK_ERR_WORKSPACE;
+  return run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws, ws_bytes, stream);
+}
+
+int do_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
+            int layout, int dtype, void* values, atk::IndexOut indices, void* ws, size_t ws_bytes,
+            hipStream_t stream) {
+  if (k < 0 || k > k0) return ATK_ERR_K;
+  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices.base);
+  if (rc != ATK_OK || k == 0 || rows == 0) return rc;
+  if (k == k0) return do_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws, ws_bytes, stream);
+  if (indices.narrow && !fits_narrow(n, k0, layout)) return ATK_ERR_TOO_LARGE;
+  {
+    bool handled = false;
+    const int rcf = atk::launch_fused_row(x, rows, n, row_stride, k0, j, k, layout, dtype, values,
+                                          indices, stream, &handled);
+    if (handled || rcf != ATK_OK) return rcf;
+  }
+  const TopkPlan p = plan_topk(rows, n, k0, j, k, layout, dtype);
+  if (!ws || ws_bytes < p.total) return ATK_ERR_WORKSPACE;
+  unsigned char* base = static_cast<unsigned char*>(ws);
+  void* cand_values = base + p.cand_values_off;
+  int64_t* cand_indices = reinterpret_cast<int64_t*>(base + p.cand_indices_off);
+  // the candidates keep int64 indices whatever the output's width
+  const int rc1 = run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, cand_values,
+                             atk::IndexOut{cand_indices, 0}, base + p.stage1_off, p.stage1_bytes, stream);
+  if (rc1 != ATK_OK) return rc1;
+  return run_select(cand_values, cand_indices, rows, k0, k, index_bound_of(n, k0, layout), dtype, values,
+                    indices, base + p.select_off, p.select_bytes, stream);
 }
 
 }  // namespace
@@ -91,7 +136,7 @@ const char* atk_strerror(int status) {
     case ATK_ERR_WORKSPACE: return "workspace missing or too small";
     case ATK_ERR_LAUNCH: return "HIP kernel launch failed";
     case ATK_ERR_ARG: return "invalid pointer or stride argument";
-    case ATK_ERR_TOO_LARGE: return "topk: too many buckets or slices";
+    case ATK_ERR_TOO_LARGE: return "topk: too many buckets or slices, or positions beyond 32-bit indices";
   }
   return "unknown status";
 }
@@ -105,10 +150,15 @@ size_t atk_stage1_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, in
 int atk_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
                int layout, int dtype, void* values, int64_t* indices, void* ws,
                size_t ws_bytes, atk_stream_t stream) {
-  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices);
-  if (rc != ATK_OK || k0 == 0 || rows == 0) return rc;
-  return run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws, ws_bytes,
-                    (hipStream_t)stream);
+  return do_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, atk::IndexOut{indices, 0}, ws,
+                   ws_bytes, (hipStream_t)stream);
+}
+
+int atk_stage1_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                   int layout, int dtype, void* values, int32_t* indices, void* ws,
+                   size_t ws_bytes, atk_stream_t stream) {
+  return do_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, atk::IndexOut{indices, 1}, ws,
+                   ws_bytes, (hipStream_t)stream);
 }
 
 size_t atk_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
@@ -122,8 +172,8 @@ int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t row
   if (rows < 0 || k0 < 0 || k < 0 || k > k0 || index_bound < 0) return ATK_ERR_K;
   if (rows == 0 || k == 0) return ATK_OK;
   if (!cand_values || !cand_indices || !values || !indices) return ATK_ERR_ARG;
-  return run_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values, indices, ws,
-                    ws_bytes, (hipStream_t)stream);
+  return run_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
+                    atk::IndexOut{indices, 0}, ws, ws_bytes, (hipStream_t)stream);
 }
 
 size_t atk_topk_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int64_t k,
@@ -134,32 +184,15 @@ size_t atk_topk_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int6
 int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
              int64_t k, int layout, int dtype, void* values, int64_t* indices, void* ws,
              size_t ws_bytes, atk_stream_t stream) {
-  if (k < 0 || k > k0) return ATK_ERR_K;
-  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices);
-  if (rc != ATK_OK || k == 0 || rows == 0) return rc;
-  if (k == k0)
-    return atk_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws,
-                      ws_bytes, stream);
-  {
-    bool handled = false;
-    const int rcf = atk::launch_fused_row(x, rows, n, row_stride, k0, j, k, layout, dtype, values,
-                                          indices, (hipStream_t)stream, &handled);
-    if (handled || rcf != ATK_OK) return rcf;
-  }
-  const TopkPlan p = plan_topk(rows, n, k0, j, k, layout, dtype);
-  if (!ws || ws_bytes < p.total) return ATK_ERR_WORKSPACE;
-  unsigned char* base = static_cast<unsigned char*>(ws);
-  void* cand_values = base + p.cand_values_off;
-  int64_t* cand_indices = reinterpret_cast<int64_t*>(base + p.cand_indices_off);
-  const int rc1 = run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, cand_values,
-                             cand_indices, base + p.stage1_off, p.stage1_bytes,
-                             (hipStream_t)stream);
-  if (rc1 != ATK_OK) return rc1;
-  const int64_t bound = (layout == ATK_CEIL_CHUNK || layout == ATK_INTERLEAVED_PADDED)
-                            ? ((n + k0 - 1) / k0) * k0
-                            : n;
-  return run_select(cand_values, cand_indices, rows, k0, k, bound, dtype, values, indices,
-                    base + p.select_off, p.select_bytes, (hipStream_t)stream);
+  return do_topk(x, rows, n, row_stride, k0, j, k, layout, dtype, values, atk::IndexOut{indices, 0}, ws,
+                 ws_bytes, (hipStream_t)stream);
+}
+
+int atk_topk_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                 int64_t k, int layout, int dtype, void* values, int32_t* indices, void* ws,
+                 size_t ws_bytes, atk_stream_t stream) {
+  return do_topk(x, rows, n, row_stride, k0, j, k, layout, dtype, values, atk::IndexOut{indices, 1}, ws,
+                 ws_bytes, (hipStream_t)stream);
 }
 
 }  // extern "C"

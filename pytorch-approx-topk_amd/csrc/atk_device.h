@@ -85,6 +85,17 @@ template <> struct Elem<ATK_I64> {
   __host__ __device__ static inline key_t key(raw_t u) { return u ^ 0x8000000000000000ull; }
 };
 
+// Destination of the result indices: int64 (the operator's contract) or, for
+// the compact entry points, int32.  `at` counts indices, not bytes.
+struct IndexOut {
+  void* base;
+  int narrow;  // != 0: int32_t
+  __device__ __forceinline__ void put(int64_t at, int64_t index) const {
+    if (narrow) static_cast<int32_t*>(base)[at] = (int32_t)index;
+    else static_cast<int64_t*>(base)[at] = index;
+  }
+};
+
 __host__ __device__ inline int elem_bytes(int dtype) {
   switch (dtype) {
     case ATK_F32: case ATK_I32: return 4;

@@ -6,12 +6,14 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "atk_device.h"
+
 namespace atk {
 
 // stage1_lane_per_bucket.hip: any dtype / layout / shape.
 int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
                                   int64_t row_stride, int64_t k0, int j, int layout,
-                                  int dtype, void* values, int64_t* indices,
+                                  int dtype, void* values, IndexOut indices,
                                   hipStream_t stream);
 
 // stage1_stream_plan.hip: interleaved layouts with at least j full sub-rows.
@@ -19,31 +21,31 @@ int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
 size_t stage1_stream_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout,
                                      int dtype);
 int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0,
-                         int j, int layout, int dtype, void* values, int64_t* indices, void* ws,
+                         int j, int layout, int dtype, void* values, IndexOut indices, void* ws,
                          size_t ws_bytes, hipStream_t stream, bool* handled);
 
 // stage1_contig_plan.hip: the contiguous layouts, through LDS.  `*handled` as above.
 size_t stage1_contig_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype);
 int launch_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                         int layout, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+                         int layout, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
                          hipStream_t stream, bool* handled);
 
 // fused_row_plan.hip: both stages in one kernel, one workgroup per row, for
 // batches of many rows whose candidates fit in LDS.  `*handled` as above.
 int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                     int64_t k, int layout, int dtype, void* values, int64_t* indices,
+                     int64_t k, int layout, int dtype, void* values, IndexOut indices,
                      hipStream_t stream, bool* handled);
 
 // stage2_radix_select.hip: one workgroup per row.
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
-                  int64_t* indices, hipStream_t stream);
+                  IndexOut indices, hipStream_t stream);
 
 // stage2_multi_select.hip: many workgroups per row, for rows with very many
 // candidates; needs a workspace.  `*handled` as above.
 size_t multi_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype);
 int launch_multi_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
-                        int64_t k, int64_t index_bound, int dtype, void* values, int64_t* indices, void* ws,
+                        int64_t k, int64_t index_bound, int dtype, void* values, IndexOut indices, void* ws,
                         size_t ws_bytes, hipStream_t stream, bool* handled);
 
 }  // namespace atk

@@ -36,7 +36,7 @@ using stream::kWave;
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
 __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) void fused_row_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
-    int64_t* __restrict__ indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t hand_off,
+    const IndexOut indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t hand_off,
     uint32_t k0, uint32_t k, int index_bits) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
       select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
 
   raw_t* ov = values + row * (int64_t)k;
-  int64_t* oi = indices + row * (int64_t)k;
+  const int64_t oi = row * (int64_t)k;  // this row's first output slot
   select::compact(
       sh, k0, k,
       [&](uint32_t i) -> bool {
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
       [&](uint32_t i) { return (int64_t)index_at(i); },
       [&](uint32_t, uint32_t o, int64_t index) {
         ov[o] = xr[index];
-        oi[o] = index;
+        indices.put(oi + o, index);
       });
 }
 
@@ -160,7 +160,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int64_t k0, int j,
-                 int64_t k, void* values, int64_t* indices, hipStream_t stream);
+                 int64_t k, void* values, IndexOut indices, hipStream_t stream);
 
 }  // namespace fused
 }  // namespace atk

@@ -8,7 +8,7 @@ namespace fused {
 
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
 static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
-                         uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+                         uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
   auto kern = fused_row_kernel<E, J, V, MAXW, pos_t, PACKED>;
   if (pl.lds_bytes > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -22,7 +22,7 @@ static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t row
 
 template <typename E, int J, int V, int MAXW, typename pos_t>
 static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
-                      uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+                      uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
   if constexpr (stream::PackedKey<E>::available && sizeof(pos_t) == 2) {
     // packed queues need every sub-row number to fit 16 bits, as pos_t == uint16_t does
     if (pl.packed) return launch_packed<E, J, V, MAXW, pos_t, true>(pl, x, rows, g, k0, k, values, indices, stream);
@@ -32,7 +32,7 @@ static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, 
 
 template <typename E, int J, int VF>
 static int launch_v(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
-                    uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+                    uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
   if (pl.waves > 8) return ATK_ERR_ARG;  // the planner never asks for more
   return pl.pos16 ? launch_one<E, J, VF, 8, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
                   : launch_one<E, J, VF, 8, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
@@ -40,7 +40,7 @@ static int launch_v(const Plan& pl, const typename E::raw_t* x, int64_t rows, co
 
 template <typename E, int J>
 static int launch_j(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
-                    uint32_t k, typename E::raw_t* values, int64_t* indices, hipStream_t stream) {
+                    uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
   constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
   if constexpr (stream::PackedKey<E>::available) {
     // packed queues may run at half the load width (fewer registers, more workgroups per CU)
@@ -51,7 +51,7 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, int64_t rows, co
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int64_t k0, int j,
-                 int64_t k, void* values, int64_t* indices, hipStream_t stream) {
+                 int64_t k, void* values, IndexOut indices, hipStream_t stream) {
   using raw_t = typename E::raw_t;
   Geom g{};
   g.row_stride = row_stride; g.b = k0 / j;
@@ -70,7 +70,7 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
 
 #define ATK_INSTANTIATE_FUSED(DT)                                                                  \
   template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int64_t, int,    \
-                                      int64_t, void*, int64_t*, hipStream_t);
+                                      int64_t, void*, IndexOut, hipStream_t);
 
 }  // namespace fused
 }  // namespace atk

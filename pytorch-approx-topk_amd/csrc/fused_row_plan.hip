@@ -86,7 +86,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
 }  // namespace fused
 
 int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                     int64_t k, int layout, int dtype, void* values, int64_t* indices, hipStream_t stream,
+                     int64_t k, int layout, int dtype, void* values, IndexOut indices, hipStream_t stream,
                      bool* handled) {
   const int es = elem_bytes(dtype);
   const int vf = es ? stream::full_vec(es) : 1;

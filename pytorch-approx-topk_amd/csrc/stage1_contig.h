@@ -84,7 +84,7 @@ template <typename E> __device__ __forceinline__ uint32_t lds_slot(uint32_t i) {
 template <typename E, int J, int V, typename F>
 __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict__ xr,
                                              typename E::raw_t* __restrict__ values,
-                                             int64_t* __restrict__ indices, void* __restrict__ partial,
+                                             const IndexOut& indices, void* __restrict__ partial,
                                              int64_t row, uint32_t group, const Geom& g, unsigned char* lds) {
   using raw_t = typename E::raw_t;
   using T = typename F::T;
@@ -238,7 +238,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
       ATK_STATIC_FOR(sl, J) {
         const uint32_t p = M::pos(acc[N - J + sl]);
         values[o + sl] = (int64_t)p < g.n ? xr[p] : E::pad_raw;
-        indices[o + sl] = p;
+        indices.put(o + sl, p);
       } ATK_STATIC_END;
     }
   }
@@ -250,7 +250,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
 template <typename E, int J, int V>
 __global__ __launch_bounds__(kThreads) void contig_kernel(const typename E::raw_t* __restrict__ x,
                                                           typename E::raw_t* __restrict__ values,
-                                                          int64_t* __restrict__ indices,
+                                                          const IndexOut indices,
                                                           void* __restrict__ partial, const Geom g) {
   extern __shared__ __align__(16) unsigned char contig_lds[];
   const uint32_t row32 = blockIdx.x / g.groups;
@@ -270,7 +270,7 @@ template <typename E, int J>
 __global__ __launch_bounds__(64) void contig_merge_kernel(const typename E::raw_t* __restrict__ x,
                                                          const void* __restrict__ partial,
                                                          typename E::raw_t* __restrict__ values,
-                                                         int64_t* __restrict__ indices, const Geom g) {
+                                                         const IndexOut indices, const Geom g) {
   using M = MergeWord<E>;
   using word_t = typename M::word_t;
   constexpr int N = J == 3 ? 4 : J;
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(64) void contig_merge_kernel(const typename E::raw_
   ATK_STATIC_FOR(sl, J) {
     const uint32_t p = M::pos(acc[N - J + sl]);
     values[o + sl] = (int64_t)p < g.n ? xr[p] : E::pad_raw;
-    indices[o + sl] = p;
+    indices.put(o + sl, p);
   } ATK_STATIC_END;
 }
 
@@ -315,7 +315,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
-                 int64_t* indices, void* ws, hipStream_t stream);
+                 IndexOut indices, void* ws, hipStream_t stream);
 
 }  // namespace contig
 }  // namespace atk

@@ -9,7 +9,7 @@ namespace contig {
 
 template <typename E, int J, int V>
 static int launch_one(const Plan& pl, const Geom& g, const typename E::raw_t* x, int64_t rows,
-                      typename E::raw_t* values, int64_t* indices, void* ws, hipStream_t stream) {
+                      typename E::raw_t* values, IndexOut indices, void* ws, hipStream_t stream) {
   const int64_t groups = rows * (int64_t)g.groups;
   if (groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   hipLaunchKernelGGL((contig_kernel<E, J, V>), dim3((unsigned)groups), dim3(kThreads), pl.lds_bytes, stream, x,
@@ -22,7 +22,7 @@ static int launch_one(const Plan& pl, const Geom& g, const typename E::raw_t* x,
 
 template <typename E, int J>
 static int launch_j(const Plan& pl, const Geom& g, const typename E::raw_t* x, int64_t rows,
-                    typename E::raw_t* values, int64_t* indices, void* ws, hipStream_t stream) {
+                    typename E::raw_t* values, IndexOut indices, void* ws, hipStream_t stream) {
   constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
   return pl.vec > 1 ? launch_one<E, J, VF>(pl, g, x, rows, values, indices, ws, stream)
                     : launch_one<E, J, 1>(pl, g, x, rows, values, indices, ws, stream);
@@ -30,7 +30,7 @@ static int launch_j(const Plan& pl, const Geom& g, const typename E::raw_t* x, i
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
-                 int64_t* indices, void* ws, hipStream_t stream) {
+                 IndexOut indices, void* ws, hipStream_t stream) {
   using raw_t = typename E::raw_t;
   Geom g = pl.geom;
   g.row_stride = row_stride;
@@ -47,7 +47,7 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
 
 #define ATK_INSTANTIATE_CONTIG(DT)                                                                \
   template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int, void*, \
-                                      int64_t*, void*, hipStream_t);
+                                      IndexOut, void*, hipStream_t);
 
 }  // namespace contig
 }  // namespace atk

@@ -82,7 +82,7 @@ size_t stage1_contig_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j,
 }
 
 int launch_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                         int layout, int dtype, void* values, int64_t* indices, void* ws, size_t ws_bytes,
+                         int layout, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
                          hipStream_t stream, bool* handled) {
   const int es = elem_bytes(dtype);
   const int vf = es ? stream::full_vec(es) : 1;

@@ -19,7 +19,7 @@ template <typename E, int J>
 __global__ __launch_bounds__(256) void stage1_lane_per_bucket_kernel(
     const typename E::raw_t* __restrict__ x, int64_t n, int64_t row_stride,
     int64_t b, int layout, int64_t blocks_per_row,
-    typename E::raw_t* __restrict__ values, int64_t* __restrict__ indices) {
+    typename E::raw_t* __restrict__ values, const IndexOut indices) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
   const int64_t row = blockIdx.x / blocks_per_row;
@@ -60,13 +60,13 @@ __global__ __launch_bounds__(256) void stage1_lane_per_bucket_kernel(
   for (int s = 0; s < J; ++s) {
     const int64_t p = pos[s];
     values[out + s] = (p >= 0 && p < n) ? xr[p] : E::pad_raw;
-    indices[out + s] = p;
+    indices.put(out + s, p);
   }
 }
 
 template <typename E>
 static int launch_for_j(const void* x, int64_t rows, int64_t n, int64_t row_stride,
-                        int64_t b, int j, int layout, void* values, int64_t* indices,
+                        int64_t b, int j, int layout, void* values, IndexOut indices,
                         hipStream_t stream) {
   using raw_t = typename E::raw_t;
   const int64_t blocks_per_row = (b + 255) / 256;
@@ -89,7 +89,7 @@ static int launch_for_j(const void* x, int64_t rows, int64_t n, int64_t row_stri
 
 int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
                                   int64_t row_stride, int64_t k0, int j, int layout,
-                                  int dtype, void* values, int64_t* indices,
+                                  int dtype, void* values, IndexOut indices,
                                   hipStream_t stream) {
   int rc = ATK_ERR_DTYPE;
   ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,

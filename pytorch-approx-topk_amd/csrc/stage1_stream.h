@@ -403,7 +403,7 @@ struct Geom {
 // queues [rows][slabs][b*J] (raw values and sub-row numbers).
 template <typename raw_t> struct Sink {
   raw_t* values;
-  int64_t* indices;
+  IndexOut indices;
   raw_t* part_values;
   uint32_t* part_pos;
 };
@@ -417,26 +417,40 @@ __device__ __forceinline__ void emit(const Geom& g, const Sink<typename E::raw_t
   if (out.part_values == nullptr) {
     const int64_t o = (row * g.b + col) * J;
     raw_t* ov = out.values + o;
-    int64_t* oi = out.indices + o;
     if constexpr (V > 1) {
       // V*J values = J stores of V elements; V*J int64 = V*J/2 16-byte stores
+      // (int32: 16-byte stores when V*J is a multiple of 4, else 8-byte ones)
       ATK_STATIC_FOR(t, J) {
         Pack<raw_t, V> pv;
         ATK_STATIC_FOR(e, V) { pv.e[e] = queue.template raw<(t * V + e) / J, (t * V + e) % J>(); } ATK_STATIC_END;
         reinterpret_cast<Pack<raw_t, V>*>(ov)[t] = pv;
       } ATK_STATIC_END;
-      ATK_STATIC_FOR(t, V * J / 2) {
-        Pack<int64_t, 2> pi;
-        ATK_STATIC_FOR(e, 2) {
-          constexpr int v = (t * 2 + e) / J, sl = (t * 2 + e) % J;
-          pi.e[e] = col + v + (int64_t)queue.template position<v, sl>() * g.b;
+      if (out.indices.narrow) {
+        constexpr int kPer = (V * J) % 4 == 0 ? 4 : 2;
+        int32_t* oi = static_cast<int32_t*>(out.indices.base) + o;
+        ATK_STATIC_FOR(t, V * J / kPer) {
+          Pack<int32_t, kPer> pi;
+          ATK_STATIC_FOR(e, kPer) {
+            constexpr int v = (t * kPer + e) / J, sl = (t * kPer + e) % J;
+            pi.e[e] = (int32_t)(col + v + (int64_t)queue.template position<v, sl>() * g.b);
+          } ATK_STATIC_END;
+          reinterpret_cast<Pack<int32_t, kPer>*>(oi)[t] = pi;
         } ATK_STATIC_END;
-        reinterpret_cast<Pack<int64_t, 2>*>(oi)[t] = pi;
-      } ATK_STATIC_END;
+      } else {
+        int64_t* oi = static_cast<int64_t*>(out.indices.base) + o;
+        ATK_STATIC_FOR(t, V * J / 2) {
+          Pack<int64_t, 2> pi;
+          ATK_STATIC_FOR(e, 2) {
+            constexpr int v = (t * 2 + e) / J, sl = (t * 2 + e) % J;
+            pi.e[e] = col + v + (int64_t)queue.template position<v, sl>() * g.b;
+          } ATK_STATIC_END;
+          reinterpret_cast<Pack<int64_t, 2>*>(oi)[t] = pi;
+        } ATK_STATIC_END;
+      }
     } else {
       ATK_STATIC_FOR(sl, J) {
         ov[sl] = queue.template raw<0, sl>();
-        oi[sl] = col + (int64_t)queue.template position<0, sl>() * g.b;
+        out.indices.put(o + sl, col + (int64_t)queue.template position<0, sl>() * g.b);
       } ATK_STATIC_END;
     }
   } else {
@@ -480,7 +494,7 @@ __device__ __forceinline__ void exact_columns(const typename E::raw_t* __restric
     if (out.part_values == nullptr) {
       const int64_t o = (row * g.b + c) * J;
 #pragma unroll
-      for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices[o + s] = c + (int64_t)pos[s] * g.b; }
+      for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices.put(o + s, c + (int64_t)pos[s] * g.b); }
     } else {
       const int64_t o = ((row * g.slabs + slab) * g.b + c) * J;
 #pragma unroll
@@ -674,7 +688,7 @@ __device__ __forceinline__ void fold_columns(const typename E::raw_t* __restrict
       ATK_STATIC_FOR(sl, J) {
         const int64_t index = c + (int64_t)M::pos(acc[N - J + sl]) * b;
         out.values[o + sl] = xr[index];
-        out.indices[o + sl] = index;
+        out.indices.put(o + sl, index);
       } ATK_STATIC_END;
     }
   }
@@ -700,7 +714,7 @@ __device__ __forceinline__ void fold_columns_exact(const typename E::raw_t* __re
     }
     const int64_t o = (row * b + c) * J;
 #pragma unroll
-    for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices[o + s] = c + (int64_t)pos[s] * b; }
+    for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices.put(o + s, c + (int64_t)pos[s] * b); }
   }
 }
 
@@ -789,7 +803,7 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
     const typename E::raw_t* __restrict__ x, int64_t row_stride,
     const typename E::raw_t* __restrict__ part_values, const uint32_t* __restrict__ part_pos,
     int64_t b, uint32_t fold, uint32_t slabs, uint32_t cb, uint32_t blocks_per_row,
-    typename E::raw_t* __restrict__ values, int64_t* __restrict__ indices) {
+    typename E::raw_t* __restrict__ values, const IndexOut indices) {
   using M = MergeWord<E>;
   using word_t = typename M::word_t;
   constexpr int N = J == 3 ? 4 : J;  // list length of the merge network
@@ -842,7 +856,7 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
   ATK_STATIC_FOR(s, J) {
     const int64_t index = c + (int64_t)M::pos(acc[N - J + s]) * b;
     values[o + s] = xr[index];
-    indices[o + s] = index;
+    indices.put(o + s, index);
   } ATK_STATIC_END;
 }
 
@@ -870,7 +884,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
 // One instance per element type, each in its own translation unit.
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
-                 int64_t* indices, void* ws, hipStream_t stream);
+                 IndexOut indices, void* ws, hipStream_t stream);
 
 }  // namespace stream
 }  // namespace atk

@@ -78,7 +78,7 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j,
-                 void* values, int64_t* indices, void* ws, hipStream_t stream) {
+                 void* values, IndexOut indices, void* ws, hipStream_t stream) {
   using raw_t = typename E::raw_t;
   Geom g;
   g.row_stride = row_stride; g.b = pl.width;
@@ -102,7 +102,7 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
 
 #define ATK_INSTANTIATE_STREAM(DT)                                                          \
   template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int, void*, \
-                                      int64_t*, void*, hipStream_t);
+                                      IndexOut, void*, hipStream_t);
 
 }  // namespace stream
 }  // namespace atk

@@ -122,12 +122,12 @@ size_t stage1_stream_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j,
 }
 
 int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                         int layout, int dtype, void* values, int64_t* indices, void* ws,
+                         int layout, int dtype, void* values, IndexOut indices, void* ws,
                          size_t ws_bytes, hipStream_t stream, bool* handled) {
   const int es = elem_bytes(dtype);
   const int vf = es ? stream::full_vec(es) : 1;
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)values % 16 == 0) &&
-                       ((uintptr_t)indices % 16 == 0) && (row_stride % vf == 0);
+                       ((uintptr_t)indices.base % 16 == 0) && (row_stride % vf == 0);
   const stream::Plan pl = stream::make_plan(rows, n, k0, j, layout, dtype, aligned);
   *handled = pl.ok;
   if (!pl.ok) return ATK_OK;

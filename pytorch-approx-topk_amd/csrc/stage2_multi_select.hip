@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kThreads) void ms_emit_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t seg, uint32_t groups, const Cut* __restrict__ cuts,
     const uint32_t* __restrict__ counts, typename E::raw_t* __restrict__ values,
-    int64_t* __restrict__ indices) {
+    const IndexOut indices) {
   __shared__ uint32_t wave_total[kWaves];
   __shared__ uint32_t start;
   const int64_t row = blockIdx.x / groups;
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kThreads) void ms_emit_kernel(
   const typename E::raw_t* cv = cand_values + row * (int64_t)k0;
   const int64_t* ci = cand_indices + row * (int64_t)k0;
   typename E::raw_t* ov = values + row * (int64_t)k;
-  int64_t* oi = indices + row * (int64_t)k;
+  const int64_t oi = row * (int64_t)k;  // this row's first output slot
   const uint32_t lo = g * seg, hi = lo + seg < k0 ? lo + seg : k0;
   const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   for (uint32_t base = lo; base < hi; base += kThreads) {
@@ -280,7 +280,7 @@ __global__ __launch_bounds__(kThreads) void ms_emit_kernel(
       const uint32_t o = out + before + rank;
       if (o < k) {  // always true for consistent inputs; keeps a wrong cut from writing out of bounds
         ov[o] = value;
-        oi[o] = ci[i];
+        indices.put(oi + o, ci[i]);
       }
     }
     out += all;
@@ -345,7 +345,7 @@ MultiPlan plan_multi(int64_t rows, int64_t k0, int64_t k, int dtype) {
 
 template <typename E>
 int launch_multi_typed(const MultiPlan& pl, const void* cand_values, const int64_t* cand_indices, int64_t rows,
-                       int64_t k0, int64_t k, int index_bits, void* values, int64_t* indices, void* ws,
+                       int64_t k0, int64_t k, int index_bits, void* values, IndexOut indices, void* ws,
                        hipStream_t stream) {
   using raw_t = typename E::raw_t;
   unsigned char* base = static_cast<unsigned char*>(ws);
@@ -384,7 +384,7 @@ size_t multi_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dty
 }
 
 int launch_multi_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
-                        int64_t k, int64_t index_bound, int dtype, void* values, int64_t* indices, void* ws,
+                        int64_t k, int64_t index_bound, int dtype, void* values, IndexOut indices, void* ws,
                         size_t ws_bytes, hipStream_t stream, bool* handled) {
   const MultiPlan pl = plan_multi(rows, k0, k, dtype);
   *handled = pl.use;

@@ -18,7 +18,7 @@ template <typename E, bool KEYS_IN_LDS>
 __global__ __launch_bounds__(1024) void select_kernel(
     const typename E::raw_t* __restrict__ cand_values,
     const int64_t* __restrict__ cand_indices, uint32_t k0, uint32_t k, int index_bits,
-    typename E::raw_t* __restrict__ values, int64_t* __restrict__ indices) {
+    typename E::raw_t* __restrict__ values, const IndexOut indices) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(1024) void select_kernel(
       select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
 
   raw_t* ov = values + row * (int64_t)k;
-  int64_t* oi = indices + row * (int64_t)k;
+  const int64_t oi = row * (int64_t)k;  // this row's first output slot
   select::compact(
       sh, k0, k,
       [&](uint32_t i) -> bool {
@@ -57,7 +57,7 @@ __global__ __launch_bounds__(1024) void select_kernel(
         return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
       },
       [&](uint32_t i) { return Candidate<raw_t>{cv[i], ci[i]}; },
-      [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) { ov[o] = c.value; oi[o] = c.index; });
+      [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) { ov[o] = c.value; indices.put(oi + o, c.index); });
 }
 
 // LDS a workgroup may use for keys; the rest of the 160 KB of a gfx950 CU is
@@ -66,7 +66,7 @@ constexpr size_t kMaxKeyLds = 128 * 1024;
 
 template <typename E>
 int launch_select_typed(const void* cand_values, const int64_t* cand_indices, int64_t rows,
-                        int64_t k0, int64_t k, int index_bits, void* values, int64_t* indices,
+                        int64_t k0, int64_t k, int index_bits, void* values, IndexOut indices,
                         hipStream_t stream) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
@@ -99,7 +99,7 @@ int launch_select_typed(const void* cand_values, const int64_t* cand_indices, in
 
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
-                  int64_t* indices, hipStream_t stream) {
+                  IndexOut indices, hipStream_t stream) {
   if (k0 > 0x7fffffffll || rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   int index_bits = 1;
   while (index_bits < 63 && (1ll << index_bits) < index_bound) ++index_bits;

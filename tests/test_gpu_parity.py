@@ -428,3 +428,42 @@ def test_gradient_scatters_to_the_selected_positions(k, j, k_mult, dim, interlea
     (x2.gather(dim, i) * w).sum().backward()
     assert torch.equal(x.grad, x2.grad)
 
+
+
+# ---- int32 indices (approx_topk.experimental.compact_indices): same results, narrower ----
+
+@pytest.mark.parametrize("rows,n,k,j,k_mult,interleaved", [
+    (6, 32768, 1024, 2, 1, True),       # streaming kernel, 16-byte index stores
+    (6, 32768, 1536, 3, 1, True),       # three entries per bucket
+    (6, 4096, 16, 1, 1, True),          # few long buckets, merged in the workgroup
+    (3, 40000, 10, 1, 1, True),         # folded and cut into slabs: merge kernel
+    (1, 1 << 20, 1024, 2, 1, True),     # slabs
+    (5, 1001, 12, 4, 1, True),          # no 16-byte loads
+    (7, 4100, 100, 2, 1, False),        # contiguous buckets
+    (3, 100003, 4, 2, 1, False),        # contiguous, chunks shared over workgroups
+    (136, 4096, 64, 1, 8, True),        # fused kernel
+    (4, 65536, 512, 2, 2, True),        # two kernels, one workgroup per row in stage 2
+    (1, 1 << 20, 32768, 1, 4, True),    # stage 2 over many workgroups
+])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.float64, torch.uint8])
+def test_int32_indices(rows, n, k, j, k_mult, interleaved, dtype):
+    from approx_topk.experimental.compact_indices import topk as topk_i32
+    x = cpu_randn((rows, n), n + k + j)
+    x = (x * 40).abs().to(dtype) if not dtype.is_floating_point else x.to(dtype)
+    xg = x.cuda()
+    v32, i32 = topk_i32(xg, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+    v64, i64 = _topk()(xg, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+    assert i32.dtype == torch.int32 and i64.dtype == torch.int64
+    assert torch.equal(i32.long(), i64)
+    assert torch.equal(v32.view(torch.uint8), v64.view(torch.uint8))
+    ev, ei = oracle_topk(x, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+    assert_same(v32, i32.long(), ev, ei, f"{dtype} rows={rows} n={n} k={k} j={j} k_mult={k_mult}")
+
+
+def test_int32_indices_refuse_rows_beyond_their_range():
+    from approx_topk.experimental.compact_indices import topk as topk_i32
+    x = torch.zeros((1, (1 << 31) + 8), dtype=torch.uint8, device="cuda")
+    with pytest.raises(RuntimeError, match="32-bit"):
+        topk_i32(x, 8, -1)
+    del x
+    torch.cuda.empty_cache()
