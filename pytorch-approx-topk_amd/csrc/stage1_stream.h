@@ -19,6 +19,19 @@
 // `slabs` along the grid; then the per-slab queues go to a workspace and
 // `stream_merge_kernel` folds them.
 //
+// Few buckets.  When the buckets do not fill one column tile, `fold`
+// consecutive sub-rows are scanned side by side as one sub-row of a matrix with
+// b*fold columns, so that every lane loads; a bucket then owns `fold` columns,
+// whose queues are merged under the full order (value, then lower index) by
+// the scanning workgroup (`fold_columns`) or by the merge kernel.
+//
+// Queues.  `CmpQueue` holds values in compare form and sub-row numbers;
+// `PackedQueue` (16-bit element types) packs an entry into one 32-bit word,
+// order key above inverted sub-row number, so that unsigned max/min/med3 insert
+// it with the right tie rule.  Register arrays are indexed by compile-time
+// constants only (ATK_STATIC_FOR): run-time indices make the compiler keep the
+// queues in scratch memory.
+//
 // Order.  Sub-rows are visited in increasing position and a newcomer displaces
 // an entry only when it compares strictly greater, so equal values keep the
 // lowest index.  Floating-point columns compare with the hardware's IEEE `>`
