@@ -72,7 +72,7 @@ int run_select(const void* cand_values, const int64_t* cand_indices, int64_t row
                                           indices, ws, ws_bytes, stream, &handled);
   if (handled || rc != ATK_OK) return rc;
   return atk::launch_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values, indices,
-                            stream);
+                            ws, ws_bytes, stream);
 }
 
 // Positions a layout can report: the row, or the padded row of the arg-max layouts.
@@ -162,7 +162,9 @@ int atk_stage1_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride, i
 }
 
 size_t atk_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
-  return atk::multi_select_workspace_bytes(rows, k0, k, dtype);
+  const size_t a = atk::multi_select_workspace_bytes(rows, k0, k, dtype);
+  const size_t b = atk::select_workspace_bytes(rows, k0, k, dtype);
+  return a > b ? a : b;
 }
 
 int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,

@@ -36,10 +36,20 @@ int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride,
                      int64_t k, int layout, int dtype, void* values, IndexOut indices,
                      hipStream_t stream, bool* handled);
 
-// stage2_radix_select.hip: one workgroup per row.
+// stage2_radix_select.hip: one workgroup per row.  With a workspace (see
+// select_workspace_bytes) and few long rows, only the cut is found by that
+// workgroup and the survivors are written by many (launch_emit_segments).
+size_t select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype);
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
-                  IndexOut indices, hipStream_t stream);
+                  IndexOut indices, void* ws, size_t ws_bytes, hipStream_t stream);
+
+// stage2_multi_select.hip: writes the survivors of every segment of `seg`
+// candidates (`groups` per row) in candidate order, given every row's cut
+// (select::GlobalCut) and the survivors counted per segment.
+int launch_emit_segments(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
+                         int64_t k, uint32_t seg, uint32_t groups, const void* cuts, const uint32_t* counts,
+                         int dtype, void* values, IndexOut indices, hipStream_t stream);
 
 // stage2_multi_select.hip: many workgroups per row, for rows with very many
 // candidates; needs a workspace.  `*handled` as above.

@@ -25,6 +25,7 @@
 // one-workgroup kernel: same survivors, same order.
 #include "atk_device.h"
 #include "atk_launch.h"
+#include "stage2_select.h"
 
 namespace atk {
 namespace {
@@ -54,7 +55,7 @@ struct State {
   uint32_t unused;
 };
 
-struct Cut { uint64_t key, index; };  // survivors: key > cut.key, or key == cut.key and index <= cut.index
+using Cut = select::GlobalCut;
 
 struct Passes {
   int key_bits, index_bits;
@@ -226,13 +227,17 @@ __global__ __launch_bounds__(kThreads) void ms_count_kernel(
   }
 }
 
+template <typename raw_t> struct Candidate { raw_t value; int64_t index; };
+struct WaveTotals { uint32_t wave_total[select::kMaxWaves]; };
+
 template <typename E>
 __global__ __launch_bounds__(kThreads) void ms_emit_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t seg, uint32_t groups, const Cut* __restrict__ cuts,
     const uint32_t* __restrict__ counts, typename E::raw_t* __restrict__ values,
     const IndexOut indices) {
-  __shared__ uint32_t wave_total[kWaves];
+  using raw_t = typename E::raw_t;
+  __shared__ WaveTotals totals;
   __shared__ uint32_t start;
   const int64_t row = blockIdx.x / groups;
   const uint32_t g = blockIdx.x - (uint32_t)row * groups;
@@ -241,50 +246,32 @@ __global__ __launch_bounds__(kThreads) void ms_emit_kernel(
   uint32_t ahead = 0;
   for (uint32_t s = threadIdx.x; s < g; s += kThreads) ahead += counts[row * groups + s];
   for (int d = kWave / 2; d >= 1; d /= 2) ahead += __shfl_down(ahead, d);
-  if (threadIdx.x % kWave == 0) wave_total[threadIdx.x / kWave] = ahead;
+  if (threadIdx.x % kWave == 0) totals.wave_total[threadIdx.x / kWave] = ahead;
   __syncthreads();
   if (threadIdx.x == 0) {
     uint32_t total = 0;
-    for (int w = 0; w < kWaves; ++w) total += wave_total[w];
+    for (int w = 0; w < kWaves; ++w) total += totals.wave_total[w];
     start = total;
   }
   __syncthreads();
-  uint32_t out = start;
+  const uint32_t first = start;
 
-  const typename E::raw_t* cv = cand_values + row * (int64_t)k0;
-  const int64_t* ci = cand_indices + row * (int64_t)k0;
-  typename E::raw_t* ov = values + row * (int64_t)k;
+  const uint32_t lo = g * seg < k0 ? g * seg : k0, hi = lo + seg < k0 ? lo + seg : k0;
+  const raw_t* cv = cand_values + row * (int64_t)k0 + lo;
+  const int64_t* ci = cand_indices + row * (int64_t)k0 + lo;
+  raw_t* ov = values + row * (int64_t)k;
   const int64_t oi = row * (int64_t)k;  // this row's first output slot
-  const uint32_t lo = g * seg, hi = lo + seg < k0 ? lo + seg : k0;
-  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  for (uint32_t base = lo; base < hi; base += kThreads) {
-    const uint32_t i = base + threadIdx.x;
-    typename E::raw_t value = 0;
-    bool keep = false;
-    if (i < hi) {
-      value = cv[i];
-      keep = survives<E>(cut, value, ci + i);
-    }
-    const uint64_t kept = __ballot(keep);
-    const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(kept >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)kept, 0u));
-    __syncthreads();  // the last round's totals are read
-    if (lane == 0) wave_total[wave] = (uint32_t)__popcll(kept);
-    __syncthreads();
-    uint32_t before = 0, all = 0;
-    for (int w = 0; w < kWaves; ++w) {
-      const uint32_t t = wave_total[w];
-      before += (uint32_t)w < wave ? t : 0u;
-      all += t;
-    }
-    if (keep) {
-      const uint32_t o = out + before + rank;
-      if (o < k) {  // always true for consistent inputs; keeps a wrong cut from writing out of bounds
-        ov[o] = value;
-        indices.put(oi + o, ci[i]);
-      }
-    }
-    out += all;
-  }
+  // the segment's survivors in candidate order, behind those of the segments before
+  select::compact(
+      totals, hi - lo, k,
+      [&](uint32_t i) -> bool { return survives<E>(cut, cv[i], ci + i); },
+      [&](uint32_t i) { return Candidate<raw_t>{cv[i], ci[i]}; },
+      [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) {
+        if (first + o < k) {  // always true for consistent inputs; keeps a wrong cut from writing out of bounds
+          ov[first + o] = c.value;
+          indices.put(oi + first + o, c.index);
+        }
+      });
 }
 
 struct MultiPlan {
@@ -377,6 +364,22 @@ int launch_multi_typed(const MultiPlan& pl, const void* cand_values, const int64
 }
 
 }  // namespace
+
+int launch_emit_segments(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
+                         int64_t k, uint32_t seg, uint32_t groups, const void* cuts, const uint32_t* counts,
+                         int dtype, void* values, IndexOut indices, hipStream_t stream) {
+  if (rows * (int64_t)groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
+  const dim3 grid((unsigned)(rows * groups)), block(kThreads);
+  int rc = ATK_ERR_DTYPE;
+  ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE, {
+    using raw_t = typename E::raw_t;
+    hipLaunchKernelGGL((ms_emit_kernel<E>), grid, block, 0, stream, static_cast<const raw_t*>(cand_values),
+                       cand_indices, (uint32_t)k0, (uint32_t)k, seg, groups, static_cast<const Cut*>(cuts), counts,
+                       static_cast<raw_t*>(values), indices);
+    rc = hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+  });
+  return rc;
+}
 
 size_t multi_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
   const MultiPlan pl = plan_multi(rows, k0, k, dtype);

@@ -18,7 +18,8 @@ template <typename E, bool KEYS_IN_LDS>
 __global__ __launch_bounds__(1024) void select_kernel(
     const typename E::raw_t* __restrict__ cand_values,
     const int64_t* __restrict__ cand_indices, uint32_t k0, uint32_t k, int index_bits,
-    typename E::raw_t* __restrict__ values, const IndexOut indices) {
+    typename E::raw_t* __restrict__ values, const IndexOut indices, select::GlobalCut* cuts,
+    uint32_t* __restrict__ counts, uint32_t seg, uint32_t groups) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
@@ -47,15 +48,41 @@ __global__ __launch_bounds__(1024) void select_kernel(
   const select::Cut<key_t> cut =
       select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
 
+  auto survives = [&](uint32_t i) -> bool {
+    const key_t key = key_at(i);
+    if (key != cut.T) return key > cut.T;
+    return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
+  };
+  if (cuts != nullptr) {
+    // Few long rows: one CU would spend as long again writing the survivors.
+    // Store the cut and the survivors of every segment of `seg` candidates;
+    // a second launch writes them with one workgroup per segment.
+    if (threadIdx.x == 0) cuts[row] = select::GlobalCut{(uint64_t)cut.T, cut.index_cut};
+    const uint32_t lane = threadIdx.x % select::kWave, wave = threadIdx.x / select::kWave;
+    const uint32_t waves = blockDim.x / select::kWave;
+    for (uint32_t g = wave; g < groups; g += waves) {
+      const uint32_t lo = g * seg < k0 ? g * seg : k0, hi = lo + seg < k0 ? lo + seg : k0;
+      uint32_t kept = 0;
+      uint32_t base = lo;
+      for (; base + 4 * select::kWave <= hi; base += 4 * select::kWave) {  // independent LDS reads
+        bool sel[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sel[u] = survives(base + u * select::kWave + lane);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) kept += (uint32_t)__popcll(__ballot(sel[u]));
+      }
+      for (; base < hi; base += select::kWave) {
+        const uint32_t i = base + lane;
+        kept += (uint32_t)__popcll(__ballot(i < hi && survives(i)));
+      }
+      if (lane == 0) counts[row * groups + g] = kept;
+    }
+    return;
+  }
   raw_t* ov = values + row * (int64_t)k;
   const int64_t oi = row * (int64_t)k;  // this row's first output slot
   select::compact(
-      sh, k0, k,
-      [&](uint32_t i) -> bool {
-        const key_t key = key_at(i);
-        if (key != cut.T) return key > cut.T;
-        return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
-      },
+      sh, k0, k, survives,
       [&](uint32_t i) { return Candidate<raw_t>{cv[i], ci[i]}; },
       [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) { ov[o] = c.value; indices.put(oi + o, c.index); });
 }
@@ -64,10 +91,32 @@ __global__ __launch_bounds__(1024) void select_kernel(
 // left to the static block above and to a second resident workgroup's needs.
 constexpr size_t kMaxKeyLds = 128 * 1024;
 
+// Few rows of many candidates each: the survivors are written by a second
+// launch, kSegments workgroups per row.
+constexpr int64_t kSplitMinCandidates = 8192;
+constexpr int64_t kSplitMaxRows = 32;
+constexpr uint32_t kSegments = 32;
+
+struct SplitPlan {
+  bool use;
+  uint32_t seg;
+  size_t counts_off, total;
+};
+
+SplitPlan plan_split(int64_t rows, int64_t k0, int64_t k) {
+  SplitPlan sp{};
+  sp.use = rows > 0 && rows <= kSplitMaxRows && k0 >= kSplitMinCandidates && k > 0 && k < k0;
+  if (!sp.use) return sp;
+  sp.seg = (uint32_t)(((k0 + kSegments - 1) / kSegments + 255) / 256 * 256);
+  sp.counts_off = ((size_t)rows * sizeof(select::GlobalCut) + 255) / 256 * 256;
+  sp.total = sp.counts_off + ((size_t)rows * kSegments * sizeof(uint32_t) + 255) / 256 * 256;
+  return sp;
+}
+
 template <typename E>
 int launch_select_typed(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                         int64_t k0, int64_t k, int index_bits, void* values, IndexOut indices,
-                        hipStream_t stream) {
+                        select::GlobalCut* cuts, uint32_t* counts, uint32_t seg, hipStream_t stream) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
   const size_t key_bytes = (size_t)k0 * sizeof(key_t);
@@ -86,28 +135,41 @@ int launch_select_typed(const void* cand_values, const int64_t* cand_indices, in
     }
     hipLaunchKernelGGL(kern, grid, block, key_bytes, stream, (const raw_t*)cand_values,
                        cand_indices, (uint32_t)k0, (uint32_t)k, index_bits, (raw_t*)values,
-                       indices);
+                       indices, cuts, counts, seg, kSegments);
   } else {
     hipLaunchKernelGGL((select_kernel<E, false>), grid, block, 0, stream,
                        (const raw_t*)cand_values, cand_indices, (uint32_t)k0, (uint32_t)k,
-                       index_bits, (raw_t*)values, indices);
+                       index_bits, (raw_t*)values, indices, cuts, counts, seg, kSegments);
   }
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
 }  // namespace
 
+size_t select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
+  (void)dtype;
+  const SplitPlan sp = plan_split(rows, k0, k);
+  return sp.use ? sp.total : 0;
+}
+
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
-                  IndexOut indices, hipStream_t stream) {
+                  IndexOut indices, void* ws, size_t ws_bytes, hipStream_t stream) {
   if (k0 > 0x7fffffffll || rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   int index_bits = 1;
   while (index_bits < 63 && (1ll << index_bits) < index_bound) ++index_bits;
+  // without a workspace the one workgroup also writes the survivors
+  const SplitPlan sp = plan_split(rows, k0, k);
+  const bool split = sp.use && ws != nullptr && ws_bytes >= sp.total && (uintptr_t)ws % 16 == 0;
+  select::GlobalCut* cuts = split ? static_cast<select::GlobalCut*>(ws) : nullptr;
+  uint32_t* counts = split ? reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(ws) + sp.counts_off) : nullptr;
   int rc = ATK_ERR_DTYPE;
   ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
-                   rc = launch_select_typed<E>(cand_values, cand_indices, rows, k0, k,
-                                               index_bits, values, indices, stream));
-  return rc;
+                   rc = launch_select_typed<E>(cand_values, cand_indices, rows, k0, k, index_bits, values,
+                                               indices, cuts, counts, sp.seg, stream));
+  if (rc != ATK_OK || !split) return rc;
+  return launch_emit_segments(cand_values, cand_indices, rows, k0, k, sp.seg, kSegments, cuts, counts, dtype,
+                              values, indices, stream);
 }
 
 }  // namespace atk

@@ -130,6 +130,10 @@ __device__ __forceinline__ void radix_pass(Sh& sh, uint32_t k0, uint32_t need, P
   __syncthreads();
 }
 
+// A row's cut as kernels hand it to one another through global memory:
+// survivors have key > cut.key, or key == cut.key and index <= cut.index.
+struct GlobalCut { uint64_t key, index; };
+
 // The cut: candidate i survives iff key(i) > T, or key(i) == T and index(i) <= index_cut.
 template <typename key_t> struct Cut {
   key_t T;
