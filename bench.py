@@ -172,7 +172,7 @@ def main() -> int:
                     help="untimed steps; the clocks of an idle GPU take ~100 launches to settle")
     ap.add_argument("--inputs", type=int, default=5, help="distinct input tensors to rotate over")
     ap.add_argument("--workload", default="C2", choices=sorted(CONFIGS))
-    ap.add_argument("--all-configs", action="store_true", help="also time C3, C4, C5 (extra JSON field)")
+    ap.add_argument("--all-configs", action="store_true", help="also time C1, C3, C4, C5 (extra JSON field)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 512 MiB device copy a few times (a kernel of known traffic for "
@@ -257,7 +257,7 @@ def main() -> int:
 
     if args.all_configs:
         others = {}
-        for other in ("C3", "C4", "C5"):
+        for other in ("C1", "C3", "C4", "C5"):
             o_rows, o_n, o_dtype, o_k, o_j, o_km, _ = CONFIGS[other]
             oxs, o_wall, o_dev_ms, o_elems, o_bytes = time_config(other, args.steps, args.warmup, args.inputs)
             o_rec, o_ok, o_checked = parity_and_recall(other, oxs[0], 2)
