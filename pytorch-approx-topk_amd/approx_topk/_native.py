@@ -95,19 +95,30 @@ def _stream(device: torch.device) -> int:
     return torch._C._cuda_getCurrentRawStream(device.index)
 
 
-class _on_device:
-    """Makes `device` current for a native call; free when it already is."""
-
-    def __init__(self, device: torch.device):
-        self.guard = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
-
+class _NoGuard:
     def __enter__(self):
-        if self.guard is not None:
-            self.guard.__enter__()
+        return None
 
     def __exit__(self, *exc):
-        if self.guard is not None:
-            self.guard.__exit__(*exc)
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on_device(device: torch.device):
+    """Makes `device` current for a native call; free when it already is."""
+    return _NO_GUARD if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+
+@functools.lru_cache(maxsize=4096)
+def _stage1_workspace(rows: int, n: int, k0: int, j: int, layout: int, code: int) -> int:
+    return lib().atk_stage1_workspace_bytes(rows, n, k0, j, layout, code)
+
+
+@functools.lru_cache(maxsize=4096)
+def _topk_workspace(rows: int, n: int, k0: int, j: int, k: int, layout: int, code: int) -> int:
+    return lib().atk_topk_workspace_bytes(rows, n, k0, j, k, layout, code)
 
 
 def rows_view(xs: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
@@ -118,6 +129,8 @@ def rows_view(xs: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
     """
     n = xs.shape[-1]
     rows = xs.numel() // n if n else 0
+    if xs.is_contiguous():  # the common case, without walking the strides
+        return xs, rows, n, n
     if xs.ndim == 1:
         return (xs if xs.stride(0) == 1 or n <= 1 else xs.contiguous()), rows, n, n
     uniform = xs.stride(-1) == 1 or n <= 1
@@ -147,7 +160,7 @@ def stage1(xs: torch.Tensor, k0: int, j: int, layout: int,
     indices = torch.empty(shape, dtype=index_dtype, device=xs.device)
     entry = L.atk_stage1 if index_dtype == torch.int64 else L.atk_stage1_i32
     with _on_device(xs.device):
-        need = L.atk_stage1_workspace_bytes(rows, n, k0, j, layout, code)
+        need = _stage1_workspace(rows, n, k0, j, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
         check(entry(xs.data_ptr(), rows, n, step, k0, j, layout, code,
                            values.data_ptr(), indices.data_ptr(),
@@ -188,7 +201,7 @@ def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int,
     indices = torch.empty(shape, dtype=index_dtype, device=xs.device)
     entry = L.atk_topk if index_dtype == torch.int64 else L.atk_topk_i32
     with _on_device(xs.device):
-        need = L.atk_topk_workspace_bytes(rows, n, k0, j, k, layout, code)
+        need = _topk_workspace(rows, n, k0, j, k, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
         check(entry(xs.data_ptr(), rows, n, step, k0, j, k, layout, code,
                          values.data_ptr(), indices.data_ptr(),
