@@ -122,8 +122,7 @@ int launch_select_typed(const void* cand_values, const int64_t* cand_indices, in
   const size_t key_bytes = (size_t)k0 * sizeof(key_t);
   const bool in_lds = key_bytes <= kMaxKeyLds;
   int nt = 1024;
-  if (k0 <= 1024) nt = 256;
-  if (k0 <= 128) nt = 64;
+  if (k0 <= 1024) nt = 512;
   const dim3 grid((unsigned)rows), block(nt);
   if (in_lds) {
     auto kern = select_kernel<E, true>;
