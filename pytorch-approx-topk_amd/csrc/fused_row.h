@@ -125,17 +125,25 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
 
   raw_t* ov = values + row * (int64_t)k;
   const int64_t oi = row * (int64_t)k;  // this row's first output slot
+  auto survives = [&](uint32_t i) -> bool {
+    const key_t key = key_at(i);
+    if (key != cut.T) return key > cut.T;
+    return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
+  };
+  // The survivors' values come from the row.  The gather is issued for every
+  // candidate of a group before any is written (those that do not survive read
+  // the row's first element), so that the loads of a group are in flight
+  // together instead of one behind each store.
+  struct Got { int64_t index; raw_t value; };
   select::compact(
-      sh, k0, k,
-      [&](uint32_t i) -> bool {
-        const key_t key = key_at(i);
-        if (key != cut.T) return key > cut.T;
-        return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
+      sh, k0, k, survives,
+      [&](uint32_t i) {
+        const int64_t index = (int64_t)index_at(i);
+        return Got{index, xr[survives(i) ? index : 0]};
       },
-      [&](uint32_t i) { return (int64_t)index_at(i); },
-      [&](uint32_t, uint32_t o, int64_t index) {
-        ov[o] = xr[index];
-        indices.put(oi + o, index);
+      [&](uint32_t, uint32_t o, const Got& got) {
+        ov[o] = got.value;
+        indices.put(oi + o, got.index);
       });
 }
 
