@@ -31,8 +31,7 @@ constexpr int kTieList = 64;
 
 template <int COPIES> struct SharedT {
   static constexpr int kCopies = COPIES;
-  uint32_t copies[COPIES * kCopyStride];
-  uint32_t hist[256];
+  uint32_t copies[COPIES * kCopyStride];  // all zero between passes
   uint32_t wave_total[kMaxWaves];
   uint32_t digit;
   uint32_t need;
@@ -55,27 +54,24 @@ __device__ __forceinline__ uint32_t rank_in(uint64_t m) {
                                    __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
 }
 
-// hist[d] = sum of the private copies of bin d
-template <typename Sh> __device__ __forceinline__ void fold_copies(Sh& sh) {
-  for (uint32_t d = threadIdx.x; d < 256; d += blockDim.x) {
-    uint32_t total = 0;
-#pragma unroll
-    for (int c = 0; c < Sh::kCopies; ++c) total += sh.copies[c * kCopyStride + d];
-    sh.hist[d] = total;
-  }
-}
-
-// Wave 0 scans the 256-bin histogram for the bin holding the `need`-th element,
-// counting from the top bin (FROM_TOP) or from the bottom bin, and publishes
-// the bin, the rank left within it and the bin's population.
+// Wave 0 sums the private copies of the 256-bin histogram (and leaves them zero
+// for the next pass), scans for the bin holding the `need`-th element, counting
+// from the top bin (FROM_TOP) or from the bottom bin, and publishes the bin,
+// the rank left within it and the bin's population.
 template <bool FROM_TOP, typename Sh>
 __device__ __forceinline__ void find_bin(Sh& sh, uint32_t need) {
   if (threadIdx.x < kWave) {
     const uint32_t lane = threadIdx.x;
     // Lane l owns bins 4l..4l+3.
-    uint32_t h[4];
+    uint32_t h[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) h[i] = sh.hist[4 * lane + i];
+    for (int c = 0; c < Sh::kCopies; ++c) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        h[i] += sh.copies[c * kCopyStride + 4 * lane + i];
+        sh.copies[c * kCopyStride + 4 * lane + i] = 0;
+      }
+    }
     const uint32_t mine = h[0] + h[1] + h[2] + h[3];
     // Inclusive scan over lanes in scan order (descending lanes when FROM_TOP).
     uint32_t incl = mine;
@@ -106,9 +102,7 @@ template <bool FROM_TOP, typename Participates, typename Sh>
 __device__ __forceinline__ void radix_pass(Sh& sh, uint32_t k0, uint32_t need, Participates digit_or_skip) {
   const uint32_t tid = threadIdx.x, nt = blockDim.x;
   uint32_t* my_copy = &sh.copies[(tid % Sh::kCopies) * kCopyStride];
-  __syncthreads();
-  for (uint32_t i = tid; i < Sh::kCopies * kCopyStride; i += nt) sh.copies[i] = 0;
-  __syncthreads();
+  __syncthreads();  // the copies are zero (clear_copies, or the last pass's find_bin)
   // four candidates per trip, so that their LDS reads and adds overlap
   uint32_t i = tid;
   for (; i + 3 * nt < k0; i += 4 * nt) {
@@ -124,10 +118,14 @@ __device__ __forceinline__ void radix_pass(Sh& sh, uint32_t k0, uint32_t need, P
     if (d >= 0) atomicAdd(&my_copy[d], 1u);
   }
   __syncthreads();
-  fold_copies(sh);
-  __syncthreads();
   find_bin<FROM_TOP>(sh, need);
   __syncthreads();
+}
+
+// Zeroes the histogram copies before the first pass (no barrier: radix_pass
+// starts with one).
+template <typename Sh> __device__ __forceinline__ void clear_copies(Sh& sh) {
+  for (uint32_t i = threadIdx.x; i < Sh::kCopies * kCopyStride; i += blockDim.x) sh.copies[i] = 0;
 }
 
 // A row's cut as kernels hand it to one another through global memory:
@@ -147,6 +145,7 @@ __device__ __forceinline__ Cut<key_t> find_cut(Sh& sh, uint32_t k0, uint32_t k, 
                                       IndexAt index_at) {
   key_t prefix = 0, mask = 0;
   uint32_t need = k;
+  clear_copies(sh);
   for (int shift = KEY_BITS - 8; shift >= 0; shift -= 8) {
     radix_pass<true>(sh, k0, need, [&](uint32_t i) -> int {
       const key_t key = key_at(i);
