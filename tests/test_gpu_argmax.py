@@ -92,3 +92,16 @@ def test_contiguous_chunks(n, k, dtype):
     ev, ei = oracle.bucketed_argmax(x, k, 1, False)
     av, ai = topk_triton(x.cuda(), k=k, dim=1, interleaved=False)
     assert_same(av, ai, ev, ei, f"n={n} k={k}")
+
+
+@pytest.mark.parametrize("layout", ["CEIL_CHUNK", "INTERLEAVED_PADDED"])
+@pytest.mark.parametrize("n,k0", [(50000, 48), (4001, 12), (100, 64), (65536, 1024)])
+def test_int32_indices_in_the_padded_layouts(layout, n, k0):
+    from approx_topk import _native
+    g = torch.Generator().manual_seed(n + k0)
+    x = torch.randn(3, n, generator=g).cuda()
+    code = getattr(_native, layout)
+    v64, i64 = _native.stage1(x, k0, 1, code)
+    v32, i32 = _native.stage1(x, k0, 1, code, torch.int32)
+    assert i32.dtype == torch.int32
+    assert torch.equal(i32.long(), i64) and torch.equal(v32, v64)
