@@ -397,8 +397,9 @@ using QueueFor = std::conditional_t<PACKED, PackedQueue<E, J, V>, CmpQueue<E, J,
 // planner folds the row: `fold` consecutive sub-rows of the true [L][b] matrix
 // form one sub-row of a matrix with b * fold columns, which is what the kernel
 // scans; column f*b + c of it holds every fold-th element of bucket c, the flat
-// index of an element is the same in both views, and the merge kernel folds the
-// `fold` columns of a bucket back together.  `b` below is the scanned width.
+// index of an element is the same in both views, and the scanning workgroup
+// folds the `fold` columns of a bucket back together.  `b` below is the scanned
+// width.
 struct Geom {
   int64_t row_stride;     // elements between rows
   int64_t b;              // columns per row as scanned
@@ -408,12 +409,13 @@ struct Geom {
   uint32_t slabs;         // sub-row slabs per row
   uint32_t slab_len;      // sub-rows per slab (the last slab takes the rest)
   uint32_t col_tiles;     // workgroup column tiles per row
-  uint32_t fold;          // > 1: the kernel itself merges the folded columns (one workgroup per row)
+  uint32_t fold;          // scanned columns per bucket (1: not folded)
 };
 
-// Where results go: final values/indices[rows][b*J], or, when the merge kernel
-// follows (several slabs, or a folded row; part_values != nullptr), per-slab
-// queues [rows][slabs][b*J] (raw values and sub-row numbers).
+// Where results go: final values/indices[rows][buckets*J], or, when the merge
+// kernel follows (several slabs; part_values != nullptr), per-slab queues
+// [rows][slabs][buckets*J] (raw values and the entries' numbers within their
+// buckets).
 template <typename raw_t> struct Sink {
   raw_t* values;
   IndexOut indices;
@@ -651,16 +653,17 @@ __device__ __forceinline__ void merge_best(typename M::word_t (&acc)[N], const t
   if constexpr (N == 2) { order(I0{}, I1{}); }
 }
 
-// The last step of a folded row that one workgroup scanned alone (wave 0, all
+// The last step of a workgroup that scanned a folded row or slab (wave 0, all
 // 64 lanes, after the waves' queues are folded): the `fold` scanned columns of
-// every bucket are merged and the final result written.  The queues go to LDS
-// as merge words; cb lanes (a power of two) then cover cb buckets at a time
-// with 64/cb lanes per bucket, which share out the bucket's columns and
-// combine pairwise by lane shuffles.
+// every bucket are merged and the bucket's entries written, as the final
+// result or as the slab's partial queue.  The queues go to LDS as merge words;
+// cb lanes (a power of two) then cover cb buckets at a time with 64/cb lanes
+// per bucket, which share out the bucket's columns and combine pairwise by
+// lane shuffles.
 template <typename E, int J, int V, typename Queue>
 __device__ __forceinline__ void fold_columns(const typename E::raw_t* __restrict__ xr, const Geom& g,
-                                             const Sink<typename E::raw_t>& out, int64_t row, int64_t col,
-                                             bool live, uint32_t lane, const Queue& queue,
+                                             const Sink<typename E::raw_t>& out, int64_t row, uint32_t slab,
+                                             int64_t col, bool live, uint32_t lane, const Queue& queue,
                                              unsigned char* lds) {
   using M = MergeWord<E>;
   using word_t = typename M::word_t;
@@ -697,37 +700,54 @@ __device__ __forceinline__ void fold_columns(const typename E::raw_t* __restrict
       merge_best<M, N>(acc, in);  // meaningful in the lanes with share < half, which are the ones read next
     }
     if (share == 0 && c < b) {
-      const int64_t o = (row * b + c) * J;
       ATK_STATIC_FOR(sl, J) {
-        const int64_t index = c + (int64_t)M::pos(acc[N - J + sl]) * b;
-        out.values[o + sl] = xr[index];
-        out.indices.put(o + sl, index);
+        const uint32_t p = M::pos(acc[N - J + sl]);  // the entry's number within its bucket
+        const int64_t index = c + (int64_t)p * b;
+        if (out.part_values == nullptr) {
+          const int64_t o = (row * b + c) * J + sl;
+          out.values[o] = xr[index];
+          out.indices.put(o, index);
+        } else {
+          const int64_t o = ((row * g.slabs + slab) * b + c) * J + sl;
+          out.part_values[o] = xr[index];
+          out.part_pos[o] = p;
+        }
       } ATK_STATIC_END;
     }
   }
 }
 
-// The same result through order keys, one lane per bucket walking the whole
-// bucket: taken when the row holds a value the fast queues cannot order.
+// The same result through order keys, one lane per bucket walking the bucket's
+// part of the scanned sub-rows [s0, s1) (and, with `tail`, what follows the
+// last full scanned sub-row): taken when the workgroup met a value the fast
+// queues cannot order.
 template <typename E, int J>
 __device__ __forceinline__ void fold_columns_exact(const typename E::raw_t* __restrict__ xr, const Geom& g,
                                                    const Sink<typename E::raw_t>& out, int64_t row,
+                                                   uint32_t slab, uint32_t s0, uint32_t s1, bool tail,
                                                    uint32_t lane) {
   using raw_t = typename E::raw_t;
   const uint32_t b = (uint32_t)g.b / g.fold;
-  const uint32_t length = g.full_rows * g.fold + g.rem / b, rem = g.rem % b;
+  const uint32_t first = s0 * g.fold;
+  const uint32_t length = s1 * g.fold + (tail ? g.rem / b : 0u), rem = tail ? g.rem % b : 0u;
   for (uint32_t c = lane; c < b; c += kWave) {
     raw_t val[J];
     uint32_t pos[J];
     clear_exact<E, J>(val, pos);
-    for (uint32_t p = 0; p < length; ++p) push_exact<E, J>(val, pos, xr[(int64_t)p * b + c], p);
+    for (uint32_t p = first; p < length; ++p) push_exact<E, J>(val, pos, xr[(int64_t)p * b + c], p);
     if (rem != 0) {
       if (c < rem) push_exact<E, J>(val, pos, xr[(int64_t)length * b + c], length);
       else if (g.pad_tail) push_exact<E, J>(val, pos, E::pad_raw, length);
     }
-    const int64_t o = (row * b + c) * J;
+    if (out.part_values == nullptr) {
+      const int64_t o = (row * b + c) * J;
 #pragma unroll
-    for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices.put(o + s, c + (int64_t)pos[s] * b); }
+      for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices.put(o + s, c + (int64_t)pos[s] * b); }
+    } else {
+      const int64_t o = ((row * g.slabs + slab) * b + c) * J;
+#pragma unroll
+      for (int s = 0; s < J; ++s) { out.part_values[o + s] = val[s]; out.part_pos[o + s] = pos[s]; }
+    }
   }
 }
 
@@ -784,10 +804,10 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
   }
   if (g.fold > 1) {
     if (redo) {
-      fold_columns_exact<E, J>(xr, g, out, row, lane);
+      fold_columns_exact<E, J>(xr, g, out, row, slab, s0, s1, last_slab, lane);
     } else {
       if (live) queue.fix_zeros(xr, g.b, col);
-      fold_columns<E, J, V>(xr, g, out, row, col, live, lane, queue, lds);
+      fold_columns<E, J, V>(xr, g, out, row, slab, col, live, lane, queue, lds);
     }
     return;
   }
@@ -800,22 +820,21 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
   emit<E, J, V>(g, out, row, slab, col, queue);
 }
 
-// Folds the partial queues of every bucket into the final result under the
-// full order (order key, then lower index).  A bucket has slabs * fold partial
-// queues ("sources"): source (slab, f) is column f*b + c of that slab's scanned
-// matrix, and its entry at scanned sub-row q is the bucket's element number
-// q*fold + f.  A workgroup of 256 threads covers `cb` buckets (a power of two
-// up to 64) with 256/cb threads per bucket, which share the sources out and
-// then combine pairwise through LDS.  Every partial queue arrives ascending,
-// so combining two is a merge network, not J insertions.  The winners' values
-// are read back from the row, so that they are the input's bit patterns.
+// Folds the slabs' partial queues of every bucket into the final result under
+// the full order (order key, then lower index); an entry's position is its
+// number within the bucket.  A workgroup of 256 threads covers `cb` buckets (a
+// power of two up to 64) with 256/cb threads per bucket, which share the slabs
+// out and then combine pairwise through LDS.  Every partial queue arrives
+// ascending, so combining two is a merge network, not J insertions.  The
+// winners' values are read back from the row, so that they are the input's bit
+// patterns.
 constexpr int kMergeThreads = 256;
 
 template <typename E, int J>
 __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
     const typename E::raw_t* __restrict__ x, int64_t row_stride,
     const typename E::raw_t* __restrict__ part_values, const uint32_t* __restrict__ part_pos,
-    int64_t b, uint32_t fold, uint32_t slabs, uint32_t cb, uint32_t blocks_per_row,
+    int64_t b, uint32_t slabs, uint32_t cb, uint32_t blocks_per_row,
     typename E::raw_t* __restrict__ values, const IndexOut indices) {
   using M = MergeWord<E>;
   using word_t = typename M::word_t;
@@ -827,27 +846,24 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
   const int64_t row = row32;
   const int64_t c = (int64_t)(blockIdx.x - row32 * blocks_per_row) * cb + t % cb;
   const bool live = c < b;
-  const int64_t width = b * fold;
   word_t acc[N], in[N];
   ATK_STATIC_FOR(s, N) { acc[s] = M::empty(); in[s] = M::empty(); } ATK_STATIC_END;
   if (live) {
-    // four sources per round, their loads issued together
+    // four slabs per round, their loads issued together
     constexpr int kBatch = 4;
-    const uint32_t sources = slabs * fold;
-    for (uint32_t src0 = share; src0 < sources; src0 += shares * kBatch) {
+    for (uint32_t slab0 = share; slab0 < slabs; slab0 += shares * kBatch) {
       typename E::raw_t got[kBatch][J];
-      uint32_t at[kBatch][J], which[kBatch];
+      uint32_t at[kBatch][J];
+      bool real[kBatch];
       ATK_STATIC_FOR(u, kBatch) {
-        const uint32_t src = src0 + u * shares;
-        const uint32_t clamped = src < sources ? src : share;  // a source that exists; ignored below
-        const uint32_t slab = clamped / fold, f = clamped - slab * fold;
-        which[u] = src < sources ? f : kEmptySlot;
-        const int64_t o = ((row * slabs + slab) * width + (int64_t)f * b + c) * J;
+        const uint32_t slab = slab0 + u * shares;
+        real[u] = slab < slabs;
+        const int64_t o = ((row * slabs + (real[u] ? slab : share)) * b + c) * J;  // a slab that exists
         ATK_STATIC_FOR(s, J) { got[u][s] = part_values[o + s]; at[u][s] = part_pos[o + s]; } ATK_STATIC_END;
       } ATK_STATIC_END;
       ATK_STATIC_FOR(u, kBatch) {
-        if (which[u] != kEmptySlot) {
-          ATK_STATIC_FOR(s, J) { in[N - J + s] = M::make(got[u][s], at[u][s] * fold + which[u]); } ATK_STATIC_END;
+        if (real[u]) {
+          ATK_STATIC_FOR(s, J) { in[N - J + s] = M::make(got[u][s], at[u][s]); } ATK_STATIC_END;
           merge_best<M, N>(acc, in);
         }
       } ATK_STATIC_END;
@@ -887,7 +903,7 @@ struct Plan {
   int64_t width;      // scanned columns per row: buckets * fold
   uint32_t full_rows, rem, pad_tail;  // of the scanned matrix
   uint32_t slabs, slab_len, col_tiles;
-  bool merge;         // the merge kernel follows (several slabs or a folded row)
+  bool merge;         // the merge kernel follows (several slabs)
   size_t part_values_off, part_pos_off, ws_bytes;
 };
 

@@ -65,14 +65,13 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
   // buckets per workgroup: a power of two, no more than there are, and few
   // enough that a thread folds at most about 32 of a bucket's partial queues
   uint32_t cb = kWave;
-  const int64_t sources = (int64_t)pl.slabs * pl.fold;
-  while (cb > 1 && ((int64_t)(cb / 2) >= b || sources * cb > 32 * kMergeThreads)) cb /= 2;
+  while (cb > 1 && ((int64_t)(cb / 2) >= b || (int64_t)pl.slabs * cb > 32 * kMergeThreads)) cb /= 2;
   const int64_t blocks_per_row = (b + cb - 1) / cb;
   if (blocks_per_row * rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)),
                      dim3(kMergeThreads), 0,
                      stream, x, g.row_stride, (const raw_t*)out.part_values, (const uint32_t*)out.part_pos,
-                     b, pl.fold, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices);
+                     b, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
@@ -84,7 +83,7 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
   g.row_stride = row_stride; g.b = pl.width;
   g.full_rows = pl.full_rows; g.rem = pl.rem; g.pad_tail = pl.pad_tail;
   g.slabs = pl.slabs; g.slab_len = pl.slab_len; g.col_tiles = pl.col_tiles;
-  g.fold = pl.merge ? 1u : pl.fold;
+  g.fold = pl.fold;
   Sink<raw_t> out;
   out.values = static_cast<raw_t*>(values); out.indices = indices;
   unsigned char* base = static_cast<unsigned char*>(ws);

@@ -12,6 +12,8 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 constexpr int64_t kTargetWaves = 1024;
 // Sub-rows worth giving to one wave before a row is also cut into slabs.
 constexpr int64_t kSlabRun = 16;
+// Sub-rows a wave keeps when a row is cut only to put a second wave on every SIMD.
+constexpr int64_t kLongRun = 64;
 // Fewest sub-rows a wave scans when several share a tile: with runs of 2 the
 // hand-over costs more than the scan (measured at 16 sub-rows: 4 waves x 4 beat
 // 8 x 2 by 25-45 %).
@@ -91,6 +93,16 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
     if (slabs > most) slabs = most;
     pl.slabs = (uint32_t)slabs;
   }
+  // Elements of one or two bytes cost twice or more the instructions per byte
+  // loaded; a second wave per SIMD hides them, while every wave still has a
+  // long run (measured on fp16 [128, 2^20] with 16 to 256 buckets: 87 -> 56 us
+  // at j = 1, 120 -> 89 us at j = 4; with shorter runs the merge eats the gain).
+  if (es <= 2) {
+    int64_t slabs = (2 * kTargetWaves + waves - 1) / waves;
+    const int64_t longest = full / (w * kLongRun);
+    if (slabs > longest) slabs = longest;
+    if (slabs > (int64_t)pl.slabs) pl.slabs = (uint32_t)slabs;
+  }
   pl.slab_len = (uint32_t)(full / pl.slabs);
   // every wave scans exactly 4 or 8 sub-rows: straight-line kernels exist for that
   pl.run = 0;
@@ -98,10 +110,11 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
     const int64_t run = full / pl.waves;
     if ((run == 4 || run == 8) && run >= j) pl.run = (int)run;
   }
-  // a folded row that one workgroup scans alone is merged by that workgroup
+  // the slabs' queues (one per bucket: a workgroup merges the folded columns of
+  // its slab itself) go to the workspace and the merge kernel follows
   pl.merge = pl.slabs > 1;
   if (pl.merge) {
-    const size_t entries = (size_t)rows * pl.slabs * (size_t)width * (size_t)j;
+    const size_t entries = (size_t)rows * pl.slabs * (size_t)b * (size_t)j;
     pl.part_values_off = 0;
     pl.part_pos_off = align_up(entries * es, 256);
     pl.ws_bytes = pl.part_pos_off + align_up(entries * sizeof(uint32_t), 256);

@@ -67,9 +67,14 @@ struct Passes {
 __device__ State advance(const State& before, const uint32_t* __restrict__ hist, int q, const Passes& ps,
                          uint32_t* lh) {
   const bool value_pass = q < ps.vc;
+  // asked for before `before` is looked at, which may still be on its way from memory
+  uint32_t mine[kBins / kThreads];
+#pragma unroll
+  for (int e = 0; e < kBins / kThreads; ++e) mine[e] = hist[e * kThreads + threadIdx.x];
   if (!value_pass && before.need == before.group) return before;  // nothing left to cut
   __shared__ State result;
-  for (uint32_t bin = threadIdx.x; bin < kBins; bin += kThreads) lh[bin] = hist[bin];
+#pragma unroll
+  for (int e = 0; e < kBins / kThreads; ++e) lh[e * kThreads + threadIdx.x] = mine[e];
   __syncthreads();
   if (threadIdx.x < kWave) {
     // value digits are searched from the top (largest keys first), index digits from the bottom
@@ -127,56 +132,76 @@ __global__ __launch_bounds__(kThreads) void ms_zero_kernel(uint32_t* words, size
   if (i < count) words[i] = 0;
 }
 
+// Candidates a thread loads ahead of testing them: the loop below is bound by
+// the latency of its loads, not by their number.
+constexpr int kBatch = 8;
+
 template <typename E>
 __global__ __launch_bounds__(kThreads) void ms_pass_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t seg, uint32_t groups, int p, const Passes ps, uint32_t* __restrict__ hist,
     State* states) {
+  using raw_t = typename E::raw_t;
   __shared__ uint32_t lh[kBins];
   const int64_t rows = gridDim.x / groups;
   const int64_t row = blockIdx.x / groups;
   const uint32_t g = blockIdx.x - (uint32_t)row * groups;
+  const raw_t* cv = cand_values + row * (int64_t)k0;
+  const int64_t* ci = cand_indices + row * (int64_t)k0;
+  const uint32_t lo = g * seg < k0 ? g * seg : k0, hi = lo + seg < k0 ? lo + seg : k0;
+  // the first batch is on its way while the state is worked out
+  auto load = [&](uint32_t base, raw_t (&into)[kBatch]) {
+#pragma unroll
+    for (int e = 0; e < kBatch; ++e) {
+      const uint32_t i = base + e * kThreads + threadIdx.x;
+      into[e] = cv[i < hi ? i : lo < k0 ? lo : 0];
+    }
+  };
+  raw_t ahead[kBatch];
+  load(lo, ahead);
+
   const State st = state_before(p, row, rows, k0, k, g == 0, ps, hist, states, lh);
   const bool value_pass = p < ps.vc;
   if (!value_pass && st.need == st.group) return;
 
   for (uint32_t bin = threadIdx.x; bin < kBins; bin += kThreads) lh[bin] = 0;
   __syncthreads();
-  const typename E::raw_t* cv = cand_values + row * (int64_t)k0;
-  const int64_t* ci = cand_indices + row * (int64_t)k0;
-  const uint32_t lo = g * seg, hi = lo + seg < k0 ? lo + seg : k0;
   const int d = value_pass ? p : p - ps.vc;
   const int shift = value_pass ? digit_shift(ps.vc, d) : digit_shift(ps.ic, d);
   const int width = value_pass ? digit_width(ps.key_bits, ps.vc, d) : digit_width(ps.index_bits, ps.ic, d);
   const uint32_t mask = (1u << width) - 1u;
+  const uint64_t prefix = value_pass ? st.key : st.index;
   const uint32_t lane = threadIdx.x % kWave;
-  for (uint32_t base = lo; base < hi; base += kThreads) {  // the same trips for every thread of a wave
-    const uint32_t i = base + threadIdx.x;
-    bool ok = i < hi;
-    uint32_t digit = 0;
-    if (ok) {
-      const uint64_t key = E::key(cv[i]);
-      if (value_pass) {
-        ok = d == 0 || (key >> (shift + width)) == st.key;
-        digit = (uint32_t)(key >> shift) & mask;
-      } else {
-        ok = key == st.key;
-        if (ok) {
-          const uint64_t index = (uint64_t)ci[i];
-          ok = d == 0 || (index >> (shift + width)) == st.index;
-          digit = (uint32_t)(index >> shift) & mask;
-        }
-      }
+  constexpr uint32_t kStep = kBatch * kThreads;
+  for (uint32_t base = lo; base < hi; base += kStep) {  // the same trips for every thread of a wave
+    raw_t now[kBatch];
+#pragma unroll
+    for (int e = 0; e < kBatch; ++e) now[e] = ahead[e];
+    if (base + kStep < hi) load(base + kStep, ahead);
+    // the number the digit is taken from: the key, or the index of a candidate with key == T
+    uint64_t from[kBatch];
+    bool ok[kBatch];
+#pragma unroll
+    for (int e = 0; e < kBatch; ++e) {
+      const uint32_t i = base + e * kThreads + threadIdx.x;
+      const uint64_t key = E::key(now[e]);
+      ok[e] = i < hi && (value_pass || key == st.key);
+      from[e] = value_pass ? key : (ok[e] ? (uint64_t)ci[i] : 0ull);
     }
-    // the leading digits of neighbouring candidates are mostly equal: count
-    // the lanes that share the first lane's digit with one atomic
-    const uint64_t live = __ballot(ok);
-    if (live != 0) {
-      const int first = __ffsll((unsigned long long)live) - 1;
-      const uint32_t lead = __shfl(digit, first);
-      const uint64_t same = __ballot(ok && digit == lead);
-      if (lane == (uint32_t)first) atomicAdd(&lh[lead], (uint32_t)__popcll(same));
-      if (ok && digit != lead) atomicAdd(&lh[digit], 1u);
+#pragma unroll
+    for (int e = 0; e < kBatch; ++e) {
+      const bool in = ok[e] && (d == 0 || (from[e] >> (shift + width)) == prefix);
+      const uint32_t digit = (uint32_t)(from[e] >> shift) & mask;
+      // the leading digits of neighbouring candidates are mostly equal: count
+      // the lanes that share the first lane's digit with one atomic
+      const uint64_t live = __ballot(in);
+      if (live != 0) {
+        const int first = __ffsll((unsigned long long)live) - 1;
+        const uint32_t lead = __shfl(digit, first);
+        const uint64_t same = __ballot(in && digit == lead);
+        if (lane == (uint32_t)first) atomicAdd(&lh[lead], (uint32_t)__popcll(same));
+        if (in && digit != lead) atomicAdd(&lh[digit], 1u);
+      }
     }
   }
   __syncthreads();
