@@ -96,6 +96,8 @@ constexpr size_t kMaxKeyLds = 128 * 1024;
 constexpr int64_t kSplitMinCandidates = 8192;
 constexpr int64_t kSplitMaxRows = 32;
 constexpr uint32_t kSegments = 32;
+// Rows from which the select is sized for throughput rather than for one row's latency.
+constexpr int64_t kManyRows = 1024;
 
 struct SplitPlan {
   bool use;
@@ -121,8 +123,16 @@ int launch_select_typed(const void* cand_values, const int64_t* cand_indices, in
   using key_t = typename E::key_t;
   const size_t key_bytes = (size_t)k0 * sizeof(key_t);
   const bool in_lds = key_bytes <= kMaxKeyLds;
+  // Few rows: as many threads as help one row finish early.  Many rows (four
+  // or more per CU): about four candidates per thread, so that more rows are
+  // resident and in different phases (measured on [4096 rows, 1024 candidates]:
+  // 38 -> 29 us; [16384, 256]: 512 threads 154 us, 64 threads 120 us in all).
   int nt = 1024;
   if (k0 <= 1024) nt = 512;
+  if (rows >= kManyRows) {
+    nt = 64;
+    while (nt < 1024 && (int64_t)nt * 4 < k0) nt *= 2;
+  }
   const dim3 grid((unsigned)rows), block(nt);
   if (in_lds) {
     auto kern = select_kernel<E, true>;

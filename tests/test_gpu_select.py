@@ -36,6 +36,7 @@ def _candidates(rows, k0, dtype, seed, ties, bound):
 @pytest.mark.parametrize("rows,k0,k", [
     (5, 64, 10), (300, 512, 64), (7, 1024, 1000), (3, 100, 100), (9, 65, 1), (130, 300, 299),
     (3, 1025, 100), (2, 40000, 777), (2, 70000, 30000),          # one workgroup per row
+    (1500, 64, 10), (1100, 256, 100), (1024, 1024, 300), (1030, 2500, 64), (2000, 40, 39),   # many rows: small workgroups
     (2, 65537, 1), (3, 131072, 32768), (1, 300001, 150000), (2, 1 << 20, 1000), (5, 100000, 99999),
 ])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.int64, torch.uint8])
