@@ -308,19 +308,17 @@ struct MultiPlan {
 };
 
 // The multi-workgroup select is taken when it is expected to be the faster one.
-// Measured on an MI355X (fp32 and fp16, k = k0/4): the chain of launches costs
-// about 45 us plus 11.7 us per million candidates of the whole batch; one
-// workgroup per row is bound by what one CU can read, about 1.2 us per thousand
-// candidates of a row (rows run side by side), until the batch as a whole is
-// bound by HBM, which the chain is as well.  Rows of up to 48K candidates
-// always stay with one workgroup (its keys then sit in LDS).
+// Measured on an MI355X (fp32 and fp16, k = k0/4, 1 to 256 rows of 64K to 4M
+// candidates): the chain of launches costs about 45 us plus 9.3 us per million
+// candidates of the whole batch; one workgroup per row is bound by what one CU
+// can read, 0.75 to 1 us per thousand candidates of a row, and slows down
+// further once more than 16 rows run side by side.  The two meet at about one
+// row per 1500 candidates of a row.  Rows of up to 48K candidates always stay
+// with one workgroup (its keys then sit in LDS).
 constexpr int64_t kMultiMinCandidates = 49152;
+constexpr int64_t kMultiCandidatesPerRow = 1500;
 
-bool multi_is_faster(int64_t rows, int64_t k0) {
-  const double multi = 45.0 + 11.7e-6 * (double)rows * (double)k0;
-  const double single = 1.2e-3 * (double)k0;
-  return multi < single;
-}
+bool multi_is_faster(int64_t rows, int64_t k0) { return rows * kMultiCandidatesPerRow <= k0; }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
