@@ -123,12 +123,14 @@ int launch_select_typed(const void* cand_values, const int64_t* cand_indices, in
   using key_t = typename E::key_t;
   const size_t key_bytes = (size_t)k0 * sizeof(key_t);
   const bool in_lds = key_bytes <= kMaxKeyLds;
-  // Few rows: as many threads as help one row finish early.  Many rows (four
-  // or more per CU): about four candidates per thread, so that more rows are
-  // resident and in different phases (measured on [4096 rows, 1024 candidates]:
-  // 38 -> 29 us; [16384, 256]: 512 threads 154 us, 64 threads 120 us in all).
+  // Few rows: as many threads as help one row finish early (256 with two
+  // histogram copies up to 1024 candidates: 5.5-8.1 us where 512 threads with
+  // eight copies take 6.1-9.1 us).  Many rows (four or more per CU): about four
+  // candidates per thread, so that more rows are resident and in different
+  // phases (measured on [4096 rows, 1024 candidates]: 38 -> 27 us; on
+  // [16384, 256]: 512 threads 99 us, 64 threads 28 us).
   int nt = 1024;
-  if (k0 <= 1024) nt = 512;
+  if (k0 <= 1024) nt = 256;
   if (rows >= kManyRows) {
     nt = 64;
     while (nt < 1024 && (int64_t)nt * 4 < k0) nt *= 2;
