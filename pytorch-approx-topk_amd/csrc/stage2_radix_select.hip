@@ -92,8 +92,10 @@ __global__ __launch_bounds__(COPIES == 8 ? 1024 : 256) void select_kernel(
 constexpr size_t kMaxKeyLds = 128 * 1024;
 
 // Few rows of many candidates each: the survivors are written by a second
-// launch, kSegments workgroups per row.
-constexpr int64_t kSplitMinCandidates = 8192;
+// launch, kSegments workgroups per row (measured per call, 1-32 rows, k = k0/4:
+// 8192 candidates 13 us in one launch, 18 us in two; 16384: 19 us either way;
+// 32768: 31 us in one, 26 us in two).
+constexpr int64_t kSplitMinCandidates = 24576;
 constexpr int64_t kSplitMaxRows = 32;
 constexpr uint32_t kSegments = 32;
 // Rows from which the select is sized for throughput rather than for one row's latency.
