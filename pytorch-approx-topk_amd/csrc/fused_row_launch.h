@@ -23,7 +23,7 @@ static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t row
 template <typename E, int J, int V, int MAXW, typename pos_t>
 static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                       uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
-  if constexpr (stream::PackedKey<E>::available && sizeof(pos_t) == 2) {
+  if constexpr (stream::PackedKey<E>::available && sizeof(typename E::raw_t) == 2 && sizeof(pos_t) == 2) {
     // packed queues need every sub-row number to fit 16 bits, as pos_t == uint16_t does
     if (pl.packed) return launch_packed<E, J, V, MAXW, pos_t, true>(pl, x, rows, g, k0, k, values, indices, stream);
   }
@@ -42,7 +42,7 @@ template <typename E, int J>
 static int launch_j(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                     uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
   constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
-  if constexpr (stream::PackedKey<E>::available) {
+  if constexpr (stream::PackedKey<E>::available && sizeof(typename E::raw_t) == 2) {
     // packed queues may run at half the load width (fewer registers, more workgroups per CU)
     if (pl.vec == VF / 2) return launch_v<E, J, VF / 2>(pl, x, rows, g, k0, k, values, indices, stream);
   }

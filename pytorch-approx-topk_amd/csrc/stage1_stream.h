@@ -26,9 +26,9 @@
 // the scanning workgroup (`fold_columns`) or by the merge kernel.
 //
 // Queues.  `CmpQueue` holds values in compare form and sub-row numbers;
-// `PackedQueue` (16-bit element types) packs an entry into one 32-bit word,
-// order key above inverted sub-row number, so that unsigned max/min/med3 insert
-// it with the right tie rule.  Register arrays are indexed by compile-time
+// `PackedQueue` (16-bit element types) and `ByteQueue` (8-bit ones) pack an
+// entry into one 32-bit word, order key above inverted sub-row number, so that
+// unsigned max/min/med3 insert it with the right tie rule.  Register arrays are indexed by compile-time
 // constants only (ATK_STATIC_FOR): run-time indices make the compiler keep the
 // queues in scratch memory.
 //
@@ -307,6 +307,18 @@ template <> struct PackedKey<Elem<ATK_I16>> {
 // largest sub-row number (the partial sub-row included) a packed entry can hold
 constexpr uint32_t kPackedMaxSubRow = 0xfffeu;
 
+// Inserts an entry word into a column's ascending words: the median of
+// (col[s], word, col[s+1]) is the new col[s].
+__device__ __forceinline__ uint32_t med3_u32(uint32_t a, uint32_t b, uint32_t c) {
+  uint32_t r;
+  asm("v_med3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+template <int J> __device__ __forceinline__ void insert_word(uint32_t (&col)[J], uint32_t word) {
+  ATK_STATIC_FOR(s, J - 1) { col[s] = med3_u32(col[s], word, col[s + 1]); } ATK_STATIC_END;
+  col[J - 1] = col[J - 1] > word ? col[J - 1] : word;
+}
+
 template <typename E, int J, int V> struct PackedQueue {
   using raw_t = typename E::raw_t;
   using K = PackedKey<E>;
@@ -322,16 +334,7 @@ template <typename E, int J, int V> struct PackedQueue {
     screen = 0;
     neg_zeros = 0;
   }
-  __device__ static __forceinline__ uint32_t med3(uint32_t a, uint32_t b, uint32_t c) {
-    uint32_t r;
-    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-  }
-  // col is ascending; the median of (col[s], word, col[s+1]) is the new col[s]
-  __device__ static __forceinline__ void insert(uint32_t (&col)[J], uint32_t word) {
-    ATK_STATIC_FOR(s, J - 1) { col[s] = med3(col[s], word, col[s + 1]); } ATK_STATIC_END;
-    col[J - 1] = col[J - 1] > word ? col[J - 1] : word;
-  }
+  __device__ static __forceinline__ void insert(uint32_t (&col)[J], uint32_t word) { insert_word<J>(col, word); }
   template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
     const uint32_t pinv = 0xffffu - p;
     if constexpr (V == 1) {
@@ -390,8 +393,71 @@ template <typename E, int J, int V> struct PackedQueue {
   template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return 0xffffu - (q[VI][SI] & 0xffffu); }
 };
 
+// The same for 8-bit element types and rows of fewer than 2^24 - 1 sub-rows:
+// the 8-bit order key in the top byte of the word, 0xFFFFFF - sub-row below it.
+// Integers have no NaN and no signed zero, so nothing is handled on the side;
+// one v_perm_b32 forms the word of an element from the loaded dword.
+template <> struct PackedKey<Elem<ATK_U8>> { static constexpr bool available = true; static constexpr uint32_t kFlip = 0u; };
+template <> struct PackedKey<Elem<ATK_I8>> { static constexpr bool available = true; static constexpr uint32_t kFlip = 0x80808080u; };
+
+// largest sub-row number (the partial sub-row included) a byte entry can hold
+constexpr uint32_t kByteMaxSubRow = 0xfffffeu;
+
+template <typename E, int J, int V> struct ByteQueue {
+  using raw_t = typename E::raw_t;
+  using K = PackedKey<E>;
+  static_assert(sizeof(raw_t) == 1 && (V % 4 == 0 || V == 1), "byte queues hold 8-bit elements");
+  static constexpr size_t kHandBytes = (size_t)V * J * kWave * 4;
+
+  uint32_t q[V][J];
+
+  __device__ __forceinline__ void reset() {
+    ATK_STATIC_FOR(e, V * J) { q[e / J][e % J] = 0; } ATK_STATIC_END;
+  }
+  __device__ static __forceinline__ void insert(uint32_t (&col)[J], uint32_t word) { insert_word<J>(col, word); }
+  template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
+    const uint32_t pinv = 0xffffffu - p;
+    if constexpr (V == 1) {
+      insert(q[0], (E::key(pk.e[0]) << 24) | pinv);
+    } else {
+      ATK_STATIC_FOR(d, V / 4) {
+        uint32_t x;  // elements 4d .. 4d+3 as loaded, lowest byte first
+        __builtin_memcpy(&x, &pk.e[4 * d], 4);
+        x ^= K::kFlip;
+        // byte 3 of the word: byte i of x; bytes 2..0: those of pinv
+        insert(q[4 * d], __builtin_amdgcn_perm(x, pinv, 0x04020100u));
+        insert(q[4 * d + 1], __builtin_amdgcn_perm(x, pinv, 0x05020100u));
+        insert(q[4 * d + 2], __builtin_amdgcn_perm(x, pinv, 0x06020100u));
+        insert(q[4 * d + 3], __builtin_amdgcn_perm(x, pinv, 0x07020100u));
+      } ATK_STATIC_END;
+    }
+  }
+  // one more element for column VI, when `valid` (the word 0 changes nothing)
+  template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
+    insert(q[VI], valid ? ((E::key(raw) << 24) | (0xffffffu - p)) : 0u);
+  }
+  __device__ __forceinline__ bool poisoned() const { return false; }
+
+  __device__ __forceinline__ void hand_over(unsigned char* area, uint32_t lane) const {
+    uint32_t* h = reinterpret_cast<uint32_t*>(area);
+    ATK_STATIC_FOR(e, V * J) { h[e * kWave + lane] = q[e / J][e % J]; } ATK_STATIC_END;
+  }
+  __device__ __forceinline__ void fold_in(const unsigned char* area, uint32_t lane) {
+    const uint32_t* h = reinterpret_cast<const uint32_t*>(area);
+    ATK_STATIC_FOR(e, V * J) { insert(q[e / J], h[e * kWave + lane]); } ATK_STATIC_END;
+  }
+  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t) {}
+  template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return q[VI][SI] >> 24; }
+  template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
+    return (raw_t)((q[VI][SI] >> 24) ^ (K::kFlip & 0xffu));
+  }
+  template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return 0xffffffu - (q[VI][SI] & 0xffffffu); }
+};
+
 template <typename E, int J, int V, bool PACKED>
-using QueueFor = std::conditional_t<PACKED, PackedQueue<E, J, V>, CmpQueue<E, J, V>>;
+using QueueFor = std::conditional_t<
+    !PACKED, CmpQueue<E, J, V>,
+    std::conditional_t<sizeof(typename E::raw_t) == 1, ByteQueue<E, J, V>, PackedQueue<E, J, V>>>;
 
 // Shape of one launch; passed to the kernels by value.  With few buckets the
 // planner folds the row: `fold` consecutive sub-rows of the true [L][b] matrix

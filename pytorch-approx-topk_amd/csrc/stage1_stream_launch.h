@@ -13,8 +13,9 @@ static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typ
   constexpr int U = J <= 2 ? 8 : 4;
   if constexpr (PackedKey<E>::available) {
     if (pl.packed) {
-      hipLaunchKernelGGL((stream_kernel<E, J, V, W, (V * J <= 8 ? 8 : 4), RUN, true>), grid, dim3(kWave * W), 0,
-                         stream, x, out, g);
+      // loads in flight: bytes load 8 per lane and keep few registers per entry
+      constexpr int UP = sizeof(typename E::raw_t) == 1 ? 8 : (V * J <= 8 ? 8 : 4);
+      hipLaunchKernelGGL((stream_kernel<E, J, V, W, UP, RUN, true>), grid, dim3(kWave * W), 0, stream, x, out, g);
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }
   }

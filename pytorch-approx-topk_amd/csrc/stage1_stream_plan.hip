@@ -54,7 +54,8 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   pl.rem = (uint32_t)(n - full * width);
   pl.pad_tail = layout == ATK_INTERLEAVED_PADDED ? 1u : 0u;
   pl.vec = (aligned && width % vf == 0) ? vf : 1;
-  pl.packed = (dtype == ATK_F16 || dtype == ATK_BF16 || dtype == ATK_I16) && full <= kPackedMaxSubRow;
+  pl.packed = ((dtype == ATK_F16 || dtype == ATK_BF16 || dtype == ATK_I16) && full <= kPackedMaxSubRow) ||
+              ((dtype == ATK_U8 || dtype == ATK_I8) && full <= kByteMaxSubRow);
 
   const int64_t tile_cols = (int64_t)kWave * pl.vec;
   pl.col_tiles = (uint32_t)((width + tile_cols - 1) / tile_cols);
