@@ -356,6 +356,20 @@ def test_few_long_buckets_special_values(dtype, n):
         _check(x, 16, -1, j=j, k_mult=km)
 
 
+@pytest.mark.parametrize("dtype", [torch.int8, torch.uint8])
+@pytest.mark.parametrize("rows,n,k,j", [
+    (2, 1 << 20, 4096, 2),      # vector loads, one packed word per entry
+    (3, 100003, 64, 4),         # odd row pitch: one column per lane
+    (1, 1 << 22, 16, 4),        # folded row cut into slabs
+    (130, 8192, 2048, 1), (5, 70001, 999, 3),
+])
+def test_byte_types_full_range(dtype, rows, n, k, j):
+    info = torch.iinfo(dtype)
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randint(info.min, info.max + 1, (rows, n), generator=g).to(dtype)   # extremes and many ties
+    _check(x, k, -1, j=j)
+
+
 def test_few_long_buckets_unaligned_rows():
     x = cpu_randn((4, 30001), 77)            # odd row pitch: no 16-byte loads
     _check(x, 16, -1, j=2)
