@@ -15,7 +15,9 @@ namespace atk {
 //   floats: IEEE value order, -0.0 == +0.0, every NaN equal and above +inf;
 //   signed integers: value order; unsigned: identity.
 // `pad_raw` is the element a padded position holds (the dtype's finite minimum,
-// as torch.finfo(dtype).min / torch.iinfo(dtype).min).
+// as torch.finfo(dtype).min / torch.iinfo(dtype).min).  `unkey` gives back the
+// element of a key where `key_is_exact` says the key names one bit pattern
+// only (not a zero, whose sign the key drops, and not a NaN).
 // ---------------------------------------------------------------------------
 template <int DT> struct Elem;
 
@@ -28,6 +30,8 @@ template <> struct Elem<ATK_F32> {
     if (u == 0x80000000u) u = 0;
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
   }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k; }
+  __host__ __device__ static inline bool key_is_exact(key_t k) { return k != 0x80000000u && k != 0xffffffffu; }
 };
 
 template <uint16_t INF, uint16_t PAD> struct Elem16Float {
@@ -39,6 +43,8 @@ template <uint16_t INF, uint16_t PAD> struct Elem16Float {
     if (u == 0x8000u) u = 0;
     return (u & 0x8000u) ? (uint16_t)~u : (uint16_t)(u | 0x8000u);
   }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return (k & 0x8000u) ? (raw_t)(k & 0x7fffu) : (raw_t)~k; }
+  __host__ __device__ static inline bool key_is_exact(key_t k) { return k != 0x8000u && k != 0xffffu; }
 };
 template <> struct Elem<ATK_F16> : Elem16Float<0x7c00u, 0xfbffu> {};
 template <> struct Elem<ATK_BF16> : Elem16Float<0x7f80u, 0xff7fu> {};
@@ -52,6 +58,8 @@ template <> struct Elem<ATK_F64> {
     if (u == 0x8000000000000000ull) u = 0;
     return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
   }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return (k >> 63) ? (k & 0x7fffffffffffffffull) : ~k; }
+  __host__ __device__ static inline bool key_is_exact(key_t k) { return k != 0x8000000000000000ull && k != ~0ull; }
 };
 
 template <> struct Elem<ATK_U8> {
@@ -59,30 +67,40 @@ template <> struct Elem<ATK_U8> {
   static constexpr int key_bits = 8;
   static constexpr raw_t pad_raw = 0;
   __host__ __device__ static inline key_t key(raw_t u) { return u; }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return (raw_t)k; }
+  __host__ __device__ static inline bool key_is_exact(key_t) { return true; }
 };
 template <> struct Elem<ATK_I8> {
   using raw_t = uint8_t; using key_t = uint32_t;
   static constexpr int key_bits = 8;
   static constexpr raw_t pad_raw = 0x80u;
   __host__ __device__ static inline key_t key(raw_t u) { return (uint8_t)(u ^ 0x80u); }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return (raw_t)(k ^ 0x80u); }
+  __host__ __device__ static inline bool key_is_exact(key_t) { return true; }
 };
 template <> struct Elem<ATK_I16> {
   using raw_t = uint16_t; using key_t = uint32_t;
   static constexpr int key_bits = 16;
   static constexpr raw_t pad_raw = 0x8000u;
   __host__ __device__ static inline key_t key(raw_t u) { return (uint16_t)(u ^ 0x8000u); }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return (raw_t)(k ^ 0x8000u); }
+  __host__ __device__ static inline bool key_is_exact(key_t) { return true; }
 };
 template <> struct Elem<ATK_I32> {
   using raw_t = uint32_t; using key_t = uint32_t;
   static constexpr int key_bits = 32;
   static constexpr raw_t pad_raw = 0x80000000u;
   __host__ __device__ static inline key_t key(raw_t u) { return u ^ 0x80000000u; }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return k ^ 0x80000000u; }
+  __host__ __device__ static inline bool key_is_exact(key_t) { return true; }
 };
 template <> struct Elem<ATK_I64> {
   using raw_t = uint64_t; using key_t = uint64_t;
   static constexpr int key_bits = 64;
   static constexpr raw_t pad_raw = 0x8000000000000000ull;
   __host__ __device__ static inline key_t key(raw_t u) { return u ^ 0x8000000000000000ull; }
+  __host__ __device__ static inline raw_t unkey(key_t k) { return k ^ 0x8000000000000000ull; }
+  __host__ __device__ static inline bool key_is_exact(key_t) { return true; }
 };
 
 // Destination of the result indices: int64 (the operator's contract) or, for

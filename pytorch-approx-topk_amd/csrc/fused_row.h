@@ -5,8 +5,9 @@
 // same register queues as the streaming stage-1 kernel (stage1_stream.h),
 // parks the k0 candidates (order key + sub-row number) in LDS, runs the
 // block-wide radix select of stage2_select.h over them and writes only the k
-// survivors, whose values it gathers from the row (still in L2) so that they
-// are the input's bit patterns.  HBM traffic is the input once plus the final
+// survivors, whose values it works out from their keys (a zero or a NaN is
+// read from the row, still in L2, so that outputs are the input's bit
+// patterns).  HBM traffic is the input once plus the final
 // k values and indices per row; the two-kernel path additionally writes and
 // re-reads k0 * (sizeof(T) + 8) bytes per row.
 //
@@ -130,16 +131,17 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
     if (key != cut.T) return key > cut.T;
     return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
   };
-  // The survivors' values come from the row.  The gather is issued for every
-  // candidate of a group before any is written (those that do not survive read
-  // the row's first element), so that the loads of a group are in flight
-  // together instead of one behind each store.
+  // The survivors' values are worked out from their keys; only a key that does
+  // not name one bit pattern (a zero, a NaN) sends its lane to the row.
   struct Got { int64_t index; raw_t value; };
   select::compact(
       sh, k0, k, survives,
       [&](uint32_t i) {
         const int64_t index = (int64_t)index_at(i);
-        return Got{index, xr[survives(i) ? index : 0]};
+        const key_t key = key_at(i);
+        raw_t value = E::unkey(key);
+        if (!E::key_is_exact(key) && survives(i)) value = xr[index];
+        return Got{index, value};
       },
       [&](uint32_t, uint32_t o, const Got& got) {
         ov[o] = got.value;

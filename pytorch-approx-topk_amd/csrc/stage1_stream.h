@@ -678,6 +678,7 @@ template <typename E, bool WIDE = (E::key_bits > 32)> struct MergeWord {
   __device__ static __forceinline__ word_t empty() { return 0; }
   __device__ static __forceinline__ bool better(word_t a, word_t b) { return a > b; }
   __device__ static __forceinline__ uint32_t pos(word_t w) { return 0xffffffffu - (uint32_t)w; }
+  __device__ static __forceinline__ typename E::key_t key(word_t w) { return (typename E::key_t)(w >> 32); }
   __device__ static __forceinline__ word_t from_lane(word_t w, int lane) { return __shfl(w, lane); }
 };
 template <typename E> struct MergeWord<E, true> {
@@ -693,10 +694,24 @@ template <typename E> struct MergeWord<E, true> {
     return a.key > b.key || (a.key == b.key && a.npos > b.npos);
   }
   __device__ static __forceinline__ uint32_t pos(const word_t& w) { return 0xffffffffu - w.npos; }
+  __device__ static __forceinline__ uint64_t key(const word_t& w) { return w.key; }
   __device__ static __forceinline__ word_t from_lane(const word_t& w, int lane) {
     return word_t{__shfl(w.key, lane), __shfl(w.npos, lane), 0u};
   }
 };
+
+// The element a merge word stands for, as the input holds it: worked out from
+// the key, or read from the row at `index` when the key does not say (a zero's
+// sign, a NaN's payload), which saves the round trip to memory in most calls.
+template <typename E>
+__device__ __forceinline__ typename E::raw_t element_of(const typename MergeWord<E>::word_t& w,
+                                                        const typename E::raw_t* __restrict__ xr,
+                                                        int64_t index) {
+  const typename E::key_t key = MergeWord<E>::key(w);
+  typename E::raw_t value = E::unkey(key);
+  if (!E::key_is_exact(key)) value = xr[index];
+  return value;
+}
 
 // acc and in are ascending lists of N entries (N a power of two); acc becomes
 // the N best of both, ascending: the element-wise better of acc and reversed
@@ -769,13 +784,14 @@ __device__ __forceinline__ void fold_columns(const typename E::raw_t* __restrict
       ATK_STATIC_FOR(sl, J) {
         const uint32_t p = M::pos(acc[N - J + sl]);  // the entry's number within its bucket
         const int64_t index = c + (int64_t)p * b;
+        const typename E::raw_t value = element_of<E>(acc[N - J + sl], xr, index);
         if (out.part_values == nullptr) {
           const int64_t o = (row * b + c) * J + sl;
-          out.values[o] = xr[index];
+          out.values[o] = value;
           out.indices.put(o, index);
         } else {
           const int64_t o = ((row * g.slabs + slab) * b + c) * J + sl;
-          out.part_values[o] = xr[index];
+          out.part_values[o] = value;
           out.part_pos[o] = p;
         }
       } ATK_STATIC_END;
@@ -892,8 +908,7 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
 // power of two up to 64) with 256/cb threads per bucket, which share the slabs
 // out and then combine pairwise through LDS.  Every partial queue arrives
 // ascending, so combining two is a merge network, not J insertions.  The
-// winners' values are read back from the row, so that they are the input's bit
-// patterns.
+// winners' values are the input's bit patterns (`element_of`).
 constexpr int kMergeThreads = 256;
 
 template <typename E, int J>
@@ -950,7 +965,7 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
   const int64_t o = (row * b + c) * J;
   ATK_STATIC_FOR(s, J) {
     const int64_t index = c + (int64_t)M::pos(acc[N - J + s]) * b;
-    values[o + s] = xr[index];
+    values[o + s] = element_of<E>(acc[N - J + s], xr, index);
     indices.put(o + s, index);
   } ATK_STATIC_END;
 }
