@@ -14,6 +14,9 @@ constexpr size_t kLdsBudget = 64 * 1024;
 // [256, 65536]: 8 beats 16 (more workgroups per CU, in different phases, and
 // cheaper barriers) and is never far behind 4.
 constexpr uint32_t kMaxWaves = 8;
+// Corners in which the two-kernel path may be the faster one (see make_plan).
+constexpr int64_t kManyRows = 1024, kAllCus = 256;
+constexpr size_t kShortRow = 128 * 1024, kLongRow = 512 * 1024;
 }  // namespace
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned) {
@@ -44,9 +47,20 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
 
   const int64_t tile_cols = (int64_t)stream::kWave * pl.vec;
   pl.tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
-  // Worth it only when parking the candidates in HBM would cost a good part of
-  // what reading the row costs: written and re-read k0*(es+8) bytes against n*es.
-  if ((size_t)k0 * (es + 8) * 4 < (size_t)n * es) return pl;
+  // One launch instead of two, and no candidates parked in HBM: measured over
+  // 128-4096 rows of 8192-262144 elements with 256-4096 candidates, this kernel
+  // is 5-40 % faster than the two-kernel path for the packed 16-bit types
+  // throughout and for wider types except in two corners: many short rows
+  // (>= 1024 rows of < 128 KiB: +5-35 %; the stand-alone select runs more rows
+  // per CU) and fewer rows than CUs with j >= 3 and rows of >= 512 KiB (+10-30 %;
+  // the two-kernel path cuts such rows into slabs).  There, and for 1-byte
+  // types (whose packed queues only the streaming kernel has), it is taken only
+  // when parking the candidates would cost a good part of what reading the row
+  // costs: written and re-read k0*(es+8) bytes against n*es.
+  const size_t row_bytes = (size_t)n * es;
+  const bool corner = es == 1 || (!pl.packed && ((rows >= kManyRows && row_bytes < kShortRow) ||
+                                                 (rows < kAllCus && j >= 3 && row_bytes >= kLongRow)));
+  if (corner && (size_t)k0 * (es + 8) * 4 < row_bytes) return pl;
   const int skey = (dtype == ATK_U8 || dtype == ATK_I8) ? 2 : es;  // stored key width
   const size_t cand_bytes = (((size_t)k0 * skey + 15) & ~(size_t)15) +
                             (((size_t)k0 * (pl.pos16 ? 2 : 4) + 15) & ~(size_t)15);
