@@ -5,8 +5,13 @@ namespace atk {
 namespace fused {
 
 namespace {
-// Rows below which one workgroup per row would leave most of the 256 CUs idle.
+// Rows below which one workgroup per row leaves most of the 256 CUs idle: taken
+// then only for rows one workgroup reads in a few microseconds, where saving
+// the second launch is what counts (1-96 rows in a HIP graph, bf16 up to 128K
+// elements: 16-31 % faster; rows of 512 KiB: even to 13 % slower; of 1 MiB: 20-60 %
+// slower).
 constexpr int64_t kMinRows = 128;
+constexpr size_t kSoloRow = 256 * 1024;
 // Dynamic LDS a workgroup may use (candidates + hand-over); the select's own
 // block adds about 9 KiB.
 constexpr size_t kLdsBudget = 64 * 1024;
@@ -24,10 +29,11 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   pl.ok = false;
   // (a padded row is never reduced further: its callers keep every bucket)
   if (layout != ATK_INTERLEAVED) return pl;
-  if (!aligned || rows < kMinRows || rows > 0x7fffffffll) return pl;
+  if (!aligned || rows > 0x7fffffffll) return pl;
   if (k0 <= 0 || k <= 0 || k >= k0 || j < 1 || j > 4 || k0 % j) return pl;
   const int es = elem_bytes(dtype);
   if (!es) return pl;
+  if (rows < kMinRows && (size_t)n * es > kSoloRow) return pl;
   const int64_t b = k0 / j;
   const int64_t full = n / b;
   if (full < j || full > 0x7fffffffll) return pl;

@@ -43,7 +43,7 @@ def test_native_argument_checks_need_no_gpu():
     assert L.atk_stage1(None, 1, 8, 8, 4, 1, 0, 0, p, p, None, 0, None) == -7  # null input
     assert L.atk_stage1(p, 1, 8, 4, 4, 1, 0, 0, p, p, None, 0, None) == -7     # row_stride < n
     assert L.atk_stage1(p, 1, 8, 8, 0, 1, 0, 0, p, p, None, 0, None) == 0      # k0 == 0: no-op
-    assert L.atk_topk(p, 1, 8, 8, 4, 1, 2, 0, 0, p, p, None, 0, None) == -5    # workspace missing
+    assert L.atk_topk(p, 1, 1 << 20, 1 << 20, 4, 1, 2, 0, 0, p, p, None, 0, None) == -5    # workspace missing (two kernels)
     assert L.atk_topk(p, 1, 8, 8, 4, 1, 5, 0, 0, p, p, None, 0, None) == -3    # k > k0
     assert L.atk_select(p, p, 1, 4, 5, 8, 0, p, p, None, 0, None) == -3
     assert L.atk_topk_workspace_bytes(3, 100, 8, 1, 8, 0, 0) == 0
