@@ -292,6 +292,9 @@ template <uint16_t INF> struct PackedKeyFloat16 {
   __device__ static __forceinline__ uint16_t unkey(uint32_t key) {
     return (uint16_t)((key & 0x8000u) ? (key ^ 0x8000u) : (0u - key));
   }
+  // the element's order key as atk_device.h defines it: negative values key one
+  // lower there (-h - 1: the complement), which leaves a gap below the zeros
+  __device__ static __forceinline__ uint32_t exact(uint32_t key) { return key - ((key >> 15) ^ 1u); }
 };
 template <> struct PackedKey<Elem<ATK_F16>> : PackedKeyFloat16<0x7c00u> {};
 template <> struct PackedKey<Elem<ATK_BF16>> : PackedKeyFloat16<0x7f80u> {};
@@ -302,6 +305,7 @@ template <> struct PackedKey<Elem<ATK_I16>> {
   __device__ static __forceinline__ uint32_t keys2(uint32_t x, uint32_t&) { return x ^ 0x80008000u; }
   __device__ static __forceinline__ bool special(uint32_t) { return false; }
   __device__ static __forceinline__ uint16_t unkey(uint32_t key) { return (uint16_t)(key ^ 0x8000u); }
+  __device__ static __forceinline__ uint32_t exact(uint32_t key) { return key; }
 };
 
 // largest sub-row number (the partial sub-row included) a packed entry can hold
@@ -383,8 +387,8 @@ template <typename E, int J, int V> struct PackedQueue {
       } ATK_STATIC_END;
     }
   }
-  // exact order key of an entry: without NaN the packed key is the exact key
-  template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return q[VI][SI] >> 16; }
+  // exact order key of an entry (the queues are not poisoned)
+  template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return K::exact(q[VI][SI] >> 16); }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
     const raw_t r = K::unkey(q[VI][SI] >> 16);
     if constexpr (K::zero_is_ambiguous) return (neg_zeros >> (VI * J + SI)) & 1u ? (raw_t)0x8000u : r;

@@ -292,6 +292,22 @@ def test_fused_rows_special_values(dtype):
         _check(x, 256, -1, j=j, k_mult=km)
 
 
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("rows,n,k,j,k_mult", [(3, 256, 128, 4, 2), (200, 256, 128, 4, 2), (130, 4096, 1024, 2, 2),
+                                               (2, 65536, 8192, 1, 4)])
+def test_fused_rows_negative_survivors(dtype, rows, n, k, j, k_mult):
+    # half or more of a row survives, so negative values are among the survivors: their
+    # values are worked out from their order keys
+    g = torch.Generator().manual_seed(rows + n)
+    if dtype.is_floating_point:
+        x = torch.randn((rows, n), generator=g).to(dtype)
+    elif dtype == torch.uint8:
+        x = torch.randint(0, 256, (rows, n), generator=g).to(dtype)
+    else:
+        x = torch.randint(-100, 100, (rows, n), generator=g).to(dtype)
+    _check(x, k, -1, j=j, k_mult=k_mult)
+
+
 def test_fused_rows_all_equal_cut_ties_by_index():
     x = torch.zeros(129, 4096)
     x[1::2] = 1.5
