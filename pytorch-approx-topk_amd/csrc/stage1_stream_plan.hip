@@ -18,9 +18,10 @@ constexpr int64_t kLongRun = 64;
 // hand-over costs more than the scan (measured at 16 sub-rows: 4 waves x 4 beat
 // 8 x 2 by 25-45 %).
 constexpr int64_t kMinRun = 4;
-// Buckets at least this long are folded when they do not fill a column tile;
-// below, merging the folded columns costs more than the idle lanes.
-constexpr int64_t kFoldMinLength = 128;
+// Buckets at least this long are folded when they do not fill a column tile
+// (measured down to 8: fp32 [32768, 1024] with 16 buckets 104 -> 22 us, bf16
+// 193 -> 32 us; [65536, 256] with 16 buckets 70 -> 31 us).
+constexpr int64_t kFoldMinLength = 8;
 }  // namespace
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned) {
@@ -36,15 +37,15 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   const int vf = full_vec(es);
 
   // Few buckets: scan `fold` sub-rows side by side so that the lanes of a wave
-  // are all busy (the largest fold that fits one column tile and keeps 16-byte
-  // loads possible); each bucket is put back together by the scanning workgroup
-  // or, when the row is also cut into slabs, by the merge kernel.
+  // are all busy (the largest fold that fits one column tile, keeps 16-byte
+  // loads possible and leaves every scanned column j elements); the scanning
+  // workgroup puts each bucket back together.
   int64_t fold = 1;
-  {
+  if (length >= kFoldMinLength) {
     const int v = aligned ? vf : 1;
     int64_t f = (int64_t)kWave * v / b;
-    while (f > 1 && (b * f) % v != 0) --f;
-    if (f > 1 && length >= kFoldMinLength && n / (b * f) >= j) fold = f;
+    while (f > 1 && ((b * f) % v != 0 || n / (b * f) < j)) --f;
+    if (f > 1) fold = f;
   }
   pl.fold = (uint32_t)fold;
   const int64_t width = b * fold;
