@@ -344,6 +344,19 @@ def test_few_long_buckets(rows, n, k, j):
     _check(cpu_randn((rows, n), n + k + j), k, -1, j=j)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8])
+@pytest.mark.parametrize("rows,n,k,j", [
+    (200, 256, 16, 1),       # buckets of 16: fold 16 (fp32), one scanned sub-row
+    (64, 1024, 64, 4),       # 16 buckets of 64, four entries each: the fold is cut down to leave 4 sub-rows
+    (33, 1000, 50, 1), (128, 640, 40, 2), (16, 512, 64, 2), (300, 2048, 32, 1), (5, 4096, 512, 1), (7, 264, 33, 1),
+])
+def test_few_short_buckets(dtype, rows, n, k, j):
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randint(0, 200, (rows, n), generator=g).to(dtype) if dtype == torch.uint8 else \
+        torch.randn((rows, n), generator=g).to(dtype)
+    _check(x, k, -1, j=j)
+
+
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
 @pytest.mark.parametrize("j,k_mult", [(1, 1), (2, 2), (3, 1), (4, 1)])
 @pytest.mark.parametrize("n", [50001, 3001])
