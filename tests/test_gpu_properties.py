@@ -135,6 +135,10 @@ def test_hip_graph_replay_matches_eager():
         (torch.randn(16, 1 << 16, device="cuda"), 1024, dict(j=2, interleaved=False)),
         (torch.randn(2, 1 << 20, device="cuda"), 8192, dict(j=2, k_mult=2)),
         (torch.randn(1, 1 << 20, device="cuda"), 32768, dict(j=1, k_mult=4)),
+        # few short rows through the fused kernel; many rows with a small select; short folded buckets
+        (torch.randn(4, 32000, device="cuda", dtype=torch.bfloat16), 64, dict(j=1, k_mult=4)),
+        (torch.randn(2048, 4096, device="cuda"), 64, dict(j=2, k_mult=4)),
+        (torch.randn(512, 1024, device="cuda"), 16, dict(j=1)),
     ]
     for _ in range(2):   # warm up allocator and library state outside the capture
         for x, k, kw in cases:
