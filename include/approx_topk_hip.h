@@ -113,6 +113,14 @@ int atk_select(const void* cand_values, const int64_t* cand_indices,
  */
 size_t atk_topk_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j,
                                 int64_t k, int layout, int dtype);
+/*
+ * The same for one particular call: 0 when the input's address and row stride
+ * let the one-kernel path take it, which parks no candidates (never more than
+ * atk_topk_workspace_bytes).  Same call site as above: the workspace the
+ * operator allocates before the native call (priority_queue.py:63-88).
+ */
+size_t atk_topk_workspace_bytes_at(const void* x, int64_t rows, int64_t n, int64_t row_stride,
+                                   int64_t k0, int j, int64_t k, int layout, int dtype);
 int atk_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride,
              int64_t k0, int j, int64_t k, int layout, int dtype,
              void* values, int64_t* indices,

@@ -19,7 +19,7 @@ DTYPE_CODE = {
     torch.uint8: 4, torch.int8: 5, torch.int16: 6, torch.int32: 7, torch.int64: 8,
 }
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 LIB_NAME = "libapprox_topk_hip.so"
 
 _SIGNATURES = {
@@ -39,6 +39,8 @@ _SIGNATURES = {
                       ctypes.c_size_t, ctypes.c_void_p]),
     "atk_topk_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 3 + [ctypes.c_int, ctypes.c_int64,
                                                                           ctypes.c_int, ctypes.c_int]),
+    "atk_topk_workspace_bytes_at": (ctypes.c_size_t, [ctypes.c_void_p] + [ctypes.c_int64] * 4
+                                    + [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]),
     "atk_topk": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4 + [ctypes.c_int, ctypes.c_int64,
                                                                            ctypes.c_int, ctypes.c_int]
                  + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
@@ -117,8 +119,10 @@ def _stage1_workspace(rows: int, n: int, k0: int, j: int, layout: int, code: int
 
 
 @functools.lru_cache(maxsize=4096)
-def _topk_workspace(rows: int, n: int, k0: int, j: int, k: int, layout: int, code: int) -> int:
-    return lib().atk_topk_workspace_bytes(rows, n, k0, j, k, layout, code)
+def _topk_workspace(misalign: int, rows: int, n: int, step: int, k0: int, j: int, k: int, layout: int,
+                    code: int) -> int:
+    # the library only looks at the address's alignment: any address with the same one stands for it
+    return lib().atk_topk_workspace_bytes_at(4096 + misalign, rows, n, step, k0, j, k, layout, code)
 
 
 def rows_view(xs: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
@@ -201,7 +205,7 @@ def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int,
     indices = torch.empty(shape, dtype=index_dtype, device=xs.device)
     entry = L.atk_topk if index_dtype == torch.int64 else L.atk_topk_i32
     with _on_device(xs.device):
-        need = _topk_workspace(rows, n, k0, j, k, layout, code)
+        need = _topk_workspace(xs.data_ptr() % 16, rows, n, step, k0, j, k, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
         check(entry(xs.data_ptr(), rows, n, step, k0, j, k, layout, code,
                          values.data_ptr(), indices.data_ptr(),

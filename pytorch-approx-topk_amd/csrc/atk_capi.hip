@@ -5,7 +5,7 @@
 
 namespace {
 
-constexpr int kAbiVersion = 1;
+constexpr int kAbiVersion = 2;
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -180,6 +180,14 @@ int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t row
 
 size_t atk_topk_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int64_t k,
                                 int layout, int dtype) {
+  return plan_topk(rows, n, k0, j, k, layout, dtype).total;
+}
+
+size_t atk_topk_workspace_bytes_at(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0,
+                                   int j, int64_t k, int layout, int dtype) {
+  if (rows > 0 && k > 0 && k < k0 && check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, x, x) == ATK_OK &&
+      atk::fused_row_takes(x, rows, n, row_stride, k0, j, k, layout, dtype))
+    return 0;
   return plan_topk(rows, n, k0, j, k, layout, dtype).total;
 }
 

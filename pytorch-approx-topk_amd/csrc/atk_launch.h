@@ -30,6 +30,10 @@ int launch_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_str
                          int layout, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
                          hipStream_t stream, bool* handled);
 
+// Whether launch_fused_row takes this very call (the input's address and row
+// stride decide with the shape).
+bool fused_row_takes(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
+                     int layout, int dtype);
 // fused_row_plan.hip: both stages in one kernel, one workgroup per row, for
 // batches of many rows whose candidates fit in LDS.  `*handled` as above.
 int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,

@@ -105,13 +105,25 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
 
 }  // namespace fused
 
-int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
-                     int64_t k, int layout, int dtype, void* values, IndexOut indices, hipStream_t stream,
-                     bool* handled) {
+namespace {
+fused::Plan plan_for(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
+                     int layout, int dtype) {
   const int es = elem_bytes(dtype);
   const int vf = es ? stream::full_vec(es) : 1;
   const bool aligned = ((uintptr_t)x % 16 == 0) && (row_stride % vf == 0);
-  const fused::Plan pl = fused::make_plan(rows, n, k0, j, k, layout, dtype, aligned);
+  return fused::make_plan(rows, n, k0, j, k, layout, dtype, aligned);
+}
+}  // namespace
+
+bool fused_row_takes(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
+                     int layout, int dtype) {
+  return plan_for(x, rows, n, row_stride, k0, j, k, layout, dtype).ok;
+}
+
+int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                     int64_t k, int layout, int dtype, void* values, IndexOut indices, hipStream_t stream,
+                     bool* handled) {
+  const fused::Plan pl = plan_for(x, rows, n, row_stride, k0, j, k, layout, dtype);
   *handled = pl.ok;
   if (!pl.ok) return ATK_OK;
   int rc = ATK_ERR_DTYPE;

@@ -28,6 +28,23 @@ def test_library_exports_every_declared_symbol():
     assert b"j must" in _native.lib().atk_strerror(-2)
 
 
+def test_workspace_of_one_call_depends_on_the_address():
+    from approx_topk import _native
+    L = _native.lib()
+    # 512 fp16 rows of 32768, 1024 candidates: one kernel, nothing parked
+    general = L.atk_topk_workspace_bytes(512, 32768, 1024, 1, 256, 0, 1)
+    assert general >= 512 * 1024 * (2 + 8)
+    assert L.atk_topk_workspace_bytes_at(4096, 512, 32768, 32768, 1024, 1, 256, 0, 1) == 0
+    # a misaligned input or an odd row stride goes through two kernels
+    assert L.atk_topk_workspace_bytes_at(4098, 512, 32768, 32768, 1024, 1, 256, 0, 1) == general
+    assert L.atk_topk_workspace_bytes_at(4096, 512, 32768, 32769, 1024, 1, 256, 0, 1) == general
+    # k == k0: stage 1 alone; contiguous buckets: never the one-kernel path
+    assert L.atk_topk_workspace_bytes_at(4096, 512, 32768, 32768, 1024, 1, 1024, 0, 1) == \
+        L.atk_topk_workspace_bytes(512, 32768, 1024, 1, 1024, 0, 1)
+    assert L.atk_topk_workspace_bytes_at(4096, 512, 32768, 32768, 1024, 1, 256, 1, 1) == \
+        L.atk_topk_workspace_bytes(512, 32768, 1024, 1, 256, 1, 1)
+
+
 def test_native_argument_checks_need_no_gpu():
     # rejected before any launch, so callable here
     from approx_topk import _native
