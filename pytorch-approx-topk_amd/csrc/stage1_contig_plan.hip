@@ -31,6 +31,10 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   g.r = (uint32_t)r;
   uint32_t lg = 0;
   while (lg < 8 && ((longest + (1ll << lg) - 1) >> lg) > piece) ++lg;
+  // Few buckets: more threads per bucket (shorter pieces, more merge rounds)
+  // as long as one workgroup still covers all of them and a piece keeps at
+  // least four elements, so that the threads of the workgroup all scan.
+  while (lg < 8 && (int64_t)(kThreads >> (lg + 1)) >= b && (m >> (lg + 1)) >= (j > 4 ? j : 4)) ++lg;
   g.pieces_log2 = lg;
   const int64_t per_thread = (longest + (1ll << lg) - 1) >> lg;
   if (per_thread > piece) {  // lg == 8: a workgroup per bucket, in chunks of 256 pieces
