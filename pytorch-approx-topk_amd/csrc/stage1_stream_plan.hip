@@ -22,6 +22,8 @@ constexpr int64_t kMinRun = 4;
 // (measured down to 8: fp32 [32768, 1024] with 16 buckets 104 -> 22 us, bf16
 // 193 -> 32 us; [65536, 256] with 16 buckets 70 -> 31 us).
 constexpr int64_t kFoldMinLength = 8;
+// Buckets from this length on are folded whatever the fold.
+constexpr int64_t kFoldAnyLength = 128;
 }  // namespace
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned) {
@@ -45,7 +47,9 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
     const int v = aligned ? vf : 1;
     int64_t f = (int64_t)kWave * v / b;
     while (f > 1 && ((b * f) % v != 0 || n / (b * f) < j)) --f;
-    if (f > 1) fold = f;
+    // short buckets: only when at least three lanes in four would idle (a fold of
+    // two costs more in the merge than it gains: [128, 4096] with 128 buckets, j = 4, +23 %)
+    if (f > 1 && (length >= kFoldAnyLength || f >= 4)) fold = f;
   }
   pl.fold = (uint32_t)fold;
   const int64_t width = b * fold;
