@@ -26,6 +26,11 @@
  *     equal and index(a) < index(b).  -0.0 equals +0.0, NaN ranks above +inf.
  *   - `ws` is caller-owned scratch of at least the matching *_workspace_bytes();
  *     it may be NULL when that size is 0.  Its contents need no initialisation.
+ *   - Alignment: the input, `values` and candidate values to the element size,
+ *     indices to their width (8 bytes; 4 for the *_i32 entry points), `ws` to
+ *     16 bytes (256 recommended); otherwise ATK_ERR_ALIGN.  Input, `values`
+ *     and `indices` that are all 16-byte aligned, with `row_stride` a multiple
+ *     of 16 bytes' worth of elements, additionally get the 16-byte-vector kernels.
  */
 #ifndef APPROX_TOPK_HIP_H_
 #define APPROX_TOPK_HIP_H_
@@ -67,7 +72,8 @@ typedef enum atk_status {
   ATK_ERR_WORKSPACE = -5,  /* ws is NULL or smaller than *_workspace_bytes() */
   ATK_ERR_LAUNCH = -6,     /* the HIP runtime rejected a launch */
   ATK_ERR_ARG = -7,        /* NULL data pointer, row_stride < n, misc. */
-  ATK_ERR_TOO_LARGE = -8   /* a size exceeds what the kernels index (cu:328,337,357) */
+  ATK_ERR_TOO_LARGE = -8,  /* a size exceeds what the kernels index (cu:328,337,357) */
+  ATK_ERR_ALIGN = -9       /* a pointer is not aligned as the conventions above require */
 } atk_status;
 
 /* Opaque hipStream_t (NULL = the default stream). */

@@ -24,6 +24,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra",
     # Packed FP32 instructions are kept out of the device code on purpose.
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # The float queues compare with the hardware's IEEE '>': subnormals must keep their
+    # order (a flush-to-zero compare would tie them with 0 and pick other candidates).
+    "-fno-gpu-flush-denormals-to-zero",
 ]
 
 

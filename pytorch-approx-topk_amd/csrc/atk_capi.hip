@@ -9,6 +9,19 @@ constexpr int kAbiVersion = 2;
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Data pointers must be aligned to what they point at (elements, indices of
+// the chosen width), a workspace to 16 bytes: the kernels carve 8-byte
+// candidate indices and 16-byte vectors out of it.
+constexpr uintptr_t kWorkspaceAlign = 16;
+inline bool aligned_to(const void* p, size_t a) { return (uintptr_t)p % a == 0; }
+int check_alignment(const void* x, const void* values, int dtype, atk::IndexOut indices, const void* ws) {
+  const size_t es = (size_t)atk::elem_bytes(dtype);
+  if (!aligned_to(x, es) || !aligned_to(values, es) || !aligned_to(indices.base, indices.narrow ? 4 : 8))
+    return ATK_ERR_ALIGN;
+  if (ws && !aligned_to(ws, kWorkspaceAlign)) return ATK_ERR_ALIGN;
+  return ATK_OK;
+}
+
 int check_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0,
                  int j, int layout, int dtype, const void* values, const void* indices) {
   if (atk::elem_bytes(dtype) == 0) return ATK_ERR_DTYPE;
@@ -88,6 +101,7 @@ int do_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_
   const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices.base);
   if (rc != ATK_OK || k0 == 0 || rows == 0) return rc;
   if (indices.narrow && !fits_narrow(n, k0, layout)) return ATK_ERR_TOO_LARGE;
+  if (const int rca = check_alignment(x, values, dtype, indices, ws); rca != ATK_OK) return rca;
   const size_t need = atk_stage1_workspace_bytes(rows, n, k0, j, layout, dtype);
   if (need && (!ws || ws_bytes < need)) return ATK_ERR_WORKSPACE;
   return run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws, ws_bytes, stream);
@@ -101,6 +115,7 @@ int do_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t 
   if (rc != ATK_OK || k == 0 || rows == 0) return rc;
   if (k == k0) return do_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices, ws, ws_bytes, stream);
   if (indices.narrow && !fits_narrow(n, k0, layout)) return ATK_ERR_TOO_LARGE;
+  if (const int rca = check_alignment(x, values, dtype, indices, ws); rca != ATK_OK) return rca;
   {
     bool handled = false;
     const int rcf = atk::launch_fused_row(x, rows, n, row_stride, k0, j, k, layout, dtype, values,
@@ -137,6 +152,8 @@ const char* atk_strerror(int status) {
     case ATK_ERR_LAUNCH: return "HIP kernel launch failed";
     case ATK_ERR_ARG: return "invalid pointer or stride argument";
     case ATK_ERR_TOO_LARGE: return "topk: too many buckets or slices, or positions beyond 32-bit indices";
+    case ATK_ERR_ALIGN:
+      return "misaligned pointer: data needs its element size, indices their width, a workspace 16 bytes";
   }
   return "unknown status";
 }
@@ -174,6 +191,9 @@ int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t row
   if (rows < 0 || k0 < 0 || k < 0 || k > k0 || index_bound < 0) return ATK_ERR_K;
   if (rows == 0 || k == 0) return ATK_OK;
   if (!cand_values || !cand_indices || !values || !indices) return ATK_ERR_ARG;
+  if (!aligned_to(cand_indices, 8)) return ATK_ERR_ALIGN;
+  if (const int rca = check_alignment(cand_values, values, dtype, atk::IndexOut{indices, 0}, ws); rca != ATK_OK)
+    return rca;
   return run_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
                     atk::IndexOut{indices, 0}, ws, ws_bytes, (hipStream_t)stream);
 }

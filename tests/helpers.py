@@ -28,3 +28,15 @@ def assert_same(got_v, got_i, exp_v, exp_i, what=""):
 
 def oracle_topk(x_cpu, k, dim=-1, j=1, k_mult=1, interleaved=True):
     return oracle.topk(x_cpu, k, dim, j=j, k_mult=k_mult, interleaved=interleaved)
+
+
+def subnormals(dtype):
+    """The smallest and largest subnormal of a float dtype and one in between, both signs,
+    next to +0.0 and -0.0: values a flush-to-zero compare would all call equal."""
+    tiny = torch.finfo(dtype).smallest_normal
+    eps = torch.finfo(dtype).eps
+    least = tiny * eps                      # smallest subnormal
+    vals = [least, 3 * least, tiny - least, 0.0]
+    t = torch.tensor(vals + [-v for v in vals], dtype=torch.float64).to(dtype)
+    assert bool(((t != 0) == torch.tensor([True] * 3 + [False] + [True] * 3 + [False])).all())
+    return t

@@ -63,6 +63,17 @@ def test_native_argument_checks_need_no_gpu():
     assert L.atk_topk(p, 1, 1 << 20, 1 << 20, 4, 1, 2, 0, 0, p, p, None, 0, None) == -5    # workspace missing (two kernels)
     assert L.atk_topk(p, 1, 8, 8, 4, 1, 5, 0, 0, p, p, None, 0, None) == -3    # k > k0
     assert L.atk_select(p, p, 1, 4, 5, 8, 0, p, p, None, 0, None) == -3
+    # misaligned pointers: data to the element size, indices to their width, workspace to 16 bytes
+    assert p % 16 == 0
+    assert L.atk_stage1(p + 2, 1, 8, 8, 4, 1, 0, 0, p, p, None, 0, None) == -9      # fp32 input at +2
+    assert L.atk_stage1(p, 1, 8, 8, 4, 1, 0, 0, p + 1, p, None, 0, None) == -9      # values
+    assert L.atk_stage1(p, 1, 8, 8, 4, 1, 0, 0, p, p + 4, None, 0, None) == -9      # int64 indices at +4
+    assert L.atk_stage1_i32(p, 1, 8, 8, 4, 1, 0, 0, p, p + 2, None, 0, None) == -9  # int32 indices at +2
+    assert L.atk_stage1(p, 1, 8, 8, 4, 1, 0, 0, p, p, p + 8, 64, None) == -9        # workspace at +8
+    assert L.atk_topk(p, 1, 1 << 20, 1 << 20, 4, 1, 2, 0, 0, p, p, p + 8, 1 << 30, None) == -9
+    assert L.atk_select(p, p + 4, 1, 4, 2, 8, 0, p, p, None, 0, None) == -9         # candidate indices
+    assert L.atk_select(p, p, 1, 4, 2, 8, 0, p, p, p + 4, 1 << 20, None) == -9
+    assert b"misaligned" in L.atk_strerror(-9)
     assert L.atk_topk_workspace_bytes(3, 100, 8, 1, 8, 0, 0) == 0
     assert L.atk_topk_workspace_bytes(3, 100, 16, 1, 8, 0, 0) >= 3 * 16 * 12
 

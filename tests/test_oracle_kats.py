@@ -291,6 +291,26 @@ def test_key_order_ints(dtype):
     assert keys == sorted(keys) and len(set(keys)) == len(keys)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+def test_subnormals_are_ordered_not_flushed(dtype):
+    from helpers import subnormals
+    t = subnormals(dtype)                   # [least, 3 least, tiny - least, +0, and their negatives]
+    keys = [oracle.key(t[i:i + 1]) for i in range(len(t))]
+    pos, neg = keys[:4], keys[4:]
+    assert pos[3] == neg[3]                 # the zeros are equal
+    assert pos[3] < pos[0] < pos[1] < pos[2]
+    assert neg[2] < neg[1] < neg[0] < neg[3]
+    # the two best of [-least, +0, +least, -0, 3 least]: 3 least (index 4) and least (index 2)
+    x = torch.stack([t[4], t[3], t[0], t[7], t[1]])
+    v, i = oracle.topk(x, 2, 0, j=2)
+    assert i.tolist() == [2, 4]             # weakest first
+    assert torch.equal(v, torch.stack([t[0], t[1]]))
+    # one bucket per element pair, interleaved: every bucket's winner is the larger subnormal
+    x = torch.stack([t[0], t[5], t[4], t[1]])       # buckets {least, -least}, {-3 least, 3 least}
+    v, i = oracle.topk(x, 2, 0, j=1)
+    assert i.tolist() == [0, 3]
+
+
 def test_nan_ranks_first_and_neg_inf_is_ordinary():
     x = torch.tensor([1.0, float("nan"), -float("inf"), 5.0, -float("inf"), 2.0])
     v, i = oracle.topk(x, 2, 0, j=2)
