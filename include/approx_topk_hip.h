@@ -73,7 +73,8 @@ typedef enum atk_status {
   ATK_ERR_LAUNCH = -6,     /* the HIP runtime rejected a launch */
   ATK_ERR_ARG = -7,        /* NULL data pointer, row_stride < n, misc. */
   ATK_ERR_TOO_LARGE = -8,  /* a size exceeds what the kernels index (cu:328,337,357) */
-  ATK_ERR_ALIGN = -9       /* a pointer is not aligned as the conventions above require */
+  ATK_ERR_ALIGN = -9,      /* a pointer is not aligned as the conventions above require */
+  ATK_ERR_SCRATCH = -10    /* atk_topk_noalloc: the call needs more than ATK_NOALLOC_SCRATCH_BYTES */
 } atk_status;
 
 /* Opaque hipStream_t (NULL = the default stream). */
@@ -148,6 +149,27 @@ int atk_topk_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride,
                  int64_t k0, int j, int64_t k, int layout, int dtype,
                  void* values, int32_t* indices,
                  void* ws, size_t ws_bytes, atk_stream_t stream);
+
+/*
+ * atk_topk without a workspace argument and without any allocation.  No
+ * counterpart in the reference: it is for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  The scratch memory atk_topk would take from the caller
+ * (stage-1 candidates, partial queues of rows cut into slabs, stage 2's
+ * histograms and counts) lives in an array of ATK_NOALLOC_SCRATCH_BYTES inside
+ * the library's device code, one copy per GPU, held until the process ends.
+ * A call that needs more (atk_topk_workspace_bytes_at() of the same arguments)
+ * returns ATK_ERR_SCRATCH and enqueues nothing.  The device the stream belongs
+ * to must be current.  All calls on one GPU share that GPU's array: calls that
+ * may run concurrently on one GPU (different streams, different host threads)
+ * race on it and must be serialised by the caller; calls on one stream are
+ * ordered and safe.  Nothing in the array needs to survive between calls and
+ * nothing needs clearing by the caller.  Results are those of atk_topk.
+ */
+#define ATK_NOALLOC_SCRATCH_BYTES ((size_t)8 << 20)
+int atk_topk_noalloc(const void* x, int64_t rows, int64_t n, int64_t row_stride,
+                     int64_t k0, int j, int64_t k, int layout, int dtype,
+                     void* values, int64_t* indices, atk_stream_t stream);
 
 #ifdef __cplusplus
 }

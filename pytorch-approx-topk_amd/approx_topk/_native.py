@@ -19,7 +19,7 @@ DTYPE_CODE = {
     torch.uint8: 4, torch.int8: 5, torch.int16: 6, torch.int32: 7, torch.int64: 8,
 }
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 LIB_NAME = "libapprox_topk_hip.so"
 
 _SIGNATURES = {
@@ -45,6 +45,9 @@ _SIGNATURES = {
                                                                            ctypes.c_int, ctypes.c_int]
                  + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
                     ctypes.c_void_p]),
+    "atk_topk_noalloc": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4
+                         + [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]
+                         + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "atk_topk_i32": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4 + [ctypes.c_int, ctypes.c_int64,
                                                                                ctypes.c_int, ctypes.c_int]
                      + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,

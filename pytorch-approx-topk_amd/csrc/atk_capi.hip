@@ -1,11 +1,38 @@
 // extern "C" entry points of libapprox_topk_hip.so: argument checks and the
 // choice of kernel.  Everything here runs on the host and only enqueues work.
+#include <mutex>
+
 #include "atk_device.h"
 #include "atk_launch.h"
 
 namespace {
 
-constexpr int kAbiVersion = 2;
+constexpr int kAbiVersion = 3;
+
+// Scratch memory of atk_topk_noalloc: one array per GPU, part of the loaded
+// code object, held until the process ends.  In host code the array's name is
+// only a handle for hipGetSymbolAddress; the device address it yields (one per
+// device) is what kernels, through do_topk's workspace argument, are given.
+constexpr size_t kScratchBytes = ATK_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// The current device's copy of `scratch`; looked up once per device.
+int scratch_of_current_device(void** out) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return ATK_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return ATK_ERR_LAUNCH;
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = g_scratch_ptr[device];
+  return ATK_OK;
+}
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -152,6 +179,9 @@ const char* atk_strerror(int status) {
     case ATK_ERR_LAUNCH: return "HIP kernel launch failed";
     case ATK_ERR_ARG: return "invalid pointer or stride argument";
     case ATK_ERR_TOO_LARGE: return "topk: too many buckets or slices, or positions beyond 32-bit indices";
+    case ATK_ERR_SCRATCH:
+      return "atk_topk_noalloc: the call needs more scratch memory than the library holds "
+             "(ATK_NOALLOC_SCRATCH_BYTES); use atk_topk with a caller workspace";
     case ATK_ERR_ALIGN:
       return "misaligned pointer: data needs its element size, indices their width, a workspace 16 bytes";
   }
@@ -223,6 +253,25 @@ int atk_topk_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride, int
                  size_t ws_bytes, atk_stream_t stream) {
   return do_topk(x, rows, n, row_stride, k0, j, k, layout, dtype, values, atk::IndexOut{indices, 1}, ws,
                  ws_bytes, (hipStream_t)stream);
+}
+
+int atk_topk_noalloc(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                     int64_t k, int layout, int dtype, void* values, int64_t* indices,
+                     atk_stream_t stream) {
+  // the checks of do_topk that decide whether any workspace is needed come first,
+  // so that an invalid call reports its own error rather than a size
+  if (k < 0 || k > k0) return ATK_ERR_K;
+  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices);
+  if (rc != ATK_OK || k == 0 || rows == 0) return rc;
+  const size_t need = atk_topk_workspace_bytes_at(x, rows, n, row_stride, k0, j, k, layout, dtype);
+  if (need > kScratchBytes) return ATK_ERR_SCRATCH;
+  void* ws = nullptr;
+  if (need != 0) {
+    const int rcs = scratch_of_current_device(&ws);
+    if (rcs != ATK_OK) return rcs;
+  }
+  return do_topk(x, rows, n, row_stride, k0, j, k, layout, dtype, values, atk::IndexOut{indices, 0}, ws,
+                 need ? kScratchBytes : 0, (hipStream_t)stream);
 }
 
 }  // extern "C"
