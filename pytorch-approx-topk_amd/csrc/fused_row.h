@@ -28,6 +28,69 @@ using stream::Cmp;
 using stream::Geom;
 using stream::kWave;
 
+// A value the fast queues cannot order (NaN) was loaded somewhere in the row:
+// stage 1 again with exact order keys, one thread per column, into the
+// candidate arrays in LDS.  All threads of the workgroup call this.
+template <typename E, int J, typename skey_t, typename pos_t>
+__device__ __forceinline__ void redo_exact_into_lds(const typename E::raw_t* __restrict__ xr, const Geom& g,
+                                                    skey_t* cand_key, pos_t* cand_pos) {
+  using raw_t = typename E::raw_t;
+  for (int64_t c = threadIdx.x; c < g.b; c += blockDim.x) {
+    raw_t qv[J];
+    uint32_t qp[J];
+    stream::clear_exact<E, J>(qv, qp);
+    for (uint32_t p = 0; p < g.full_rows; ++p) stream::push_exact<E, J>(qv, qp, xr[(int64_t)p * g.b + c], p);
+    if (g.rem != 0) {
+      if (c < (int64_t)g.rem)
+        stream::push_exact<E, J>(qv, qp, xr[(int64_t)g.full_rows * g.b + c], g.full_rows);
+      else if (g.pad_tail)
+        stream::push_exact<E, J>(qv, qp, E::pad_raw, g.full_rows);
+    }
+#pragma unroll
+    for (int s = 0; s < J; ++s) { cand_key[c * J + s] = (skey_t)E::key(qv[s]); cand_pos[c * J + s] = (pos_t)qp[s]; }
+  }
+}
+
+// Stage 2 over the candidates parked in LDS (exact order keys and sub-row
+// numbers, candidate c*J + s belonging to column c): the block-wide radix
+// select, then the survivors in candidate order.  Starts with a barrier.
+template <typename E, int J, typename skey_t, typename pos_t, typename Sh>
+__device__ __forceinline__ void select_from_lds(Sh& sh, const typename E::raw_t* __restrict__ xr, const Geom& g,
+                                                const skey_t* cand_key, const pos_t* cand_pos, uint32_t k0,
+                                                uint32_t k, int index_bits, int64_t row,
+                                                typename E::raw_t* __restrict__ values, const IndexOut& indices) {
+  using raw_t = typename E::raw_t;
+  using key_t = typename E::key_t;
+  auto key_at = [&](uint32_t i) -> key_t { return cand_key[i]; };
+  auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)cand_pos[i] * (uint64_t)g.b + i / J; };
+  const select::Cut<key_t> cut =
+      select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
+
+  raw_t* ov = values + row * (int64_t)k;
+  const int64_t oi = row * (int64_t)k;  // this row's first output slot
+  auto survives = [&](uint32_t i) -> bool {
+    const key_t key = key_at(i);
+    if (key != cut.T) return key > cut.T;
+    return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
+  };
+  // The survivors' values are worked out from their keys; only a key that does
+  // not name one bit pattern (a zero, a NaN) sends its lane to the row.
+  struct Got { int64_t index; raw_t value; };
+  select::compact(
+      sh, k0, k, survives,
+      [&](uint32_t i) {
+        const int64_t index = (int64_t)index_at(i);
+        const key_t key = key_at(i);
+        raw_t value = E::unkey(key);
+        if (!E::key_is_exact(key) && survives(i)) value = xr[index];
+        return Got{index, value};
+      },
+      [&](uint32_t, uint32_t o, const Got& got) {
+        ov[o] = got.value;
+        indices.put(oi + o, got.index);
+      });
+}
+
 // pos_t: uint16_t when every sub-row number fits, else uint32_t.  PACKED: packed
 // 16-bit queues (stage1_stream.h).
 // The SGPR cap keeps eight waves per SIMD possible (beyond 96 scalar registers
@@ -99,54 +162,384 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
     if (split > 1 && hand_off != 0) __syncthreads();  // the hand-over area is reused by the next round
   }
 
-  if (__syncthreads_or(any_nan)) {
-    // a value the fast queues cannot order (NaN; -0.0 for packed queues) was
-    // loaded somewhere in the row: redo stage 1 with exact order keys
-    for (int64_t c = threadIdx.x; c < g.b; c += blockDim.x) {
-      raw_t qv[J];
-      uint32_t qp[J];
-      stream::clear_exact<E, J>(qv, qp);
-      for (uint32_t p = 0; p < g.full_rows; ++p) stream::push_exact<E, J>(qv, qp, xr[(int64_t)p * g.b + c], p);
-      if (g.rem != 0) {
-        if (c < (int64_t)g.rem)
-          stream::push_exact<E, J>(qv, qp, xr[(int64_t)g.full_rows * g.b + c], g.full_rows);
-        else if (g.pad_tail)
-          stream::push_exact<E, J>(qv, qp, E::pad_raw, g.full_rows);
-      }
+  if (__syncthreads_or(any_nan)) redo_exact_into_lds<E, J>(xr, g, cand_key, cand_pos);
+  // (the select's first pass starts with a barrier, which also publishes the candidates)
+  select_from_lds<E, J>(sh, xr, g, cand_key, cand_pos, k0, k, index_bits, row, values, indices);
+}
+
+// ---------------------------------------------------------------------------
+// The same with the candidates kept in registers through stage 2, for rows all
+// of whose column tiles are scanned at once (tiles * split <= waves): when the
+// scan ends, every lane of a tile's leading wave holds its V*J candidates, so
+// nothing is parked in LDS.  The cut is found by an MSB-first radix select with
+// 12-bit digits whose histograms (4096 bins in LDS, one atomic add per
+// candidate straight from its register) are read by all threads; as soon as
+// the bin that holds the k-th best has at most kListMax members, those are
+// listed and ranked under the full order (key, then lower index), which gives
+// the cut in one step whatever key bits are left.  Survivors are counted per
+// lane, placed by a wave prefix sum and per-wave bases, and written from
+// registers in candidate order.  Rows that met a NaN, or whose cut falls among
+// more than kListMax candidates with one and the same key, take the LDS path
+// of the kernel above.  Results are identical.
+// ---------------------------------------------------------------------------
+namespace regs {
+
+constexpr int kDigitBits = 11;
+constexpr int kBins = 1 << kDigitBits;
+constexpr uint32_t kListMax = 64;
+
+// A histogram holds the count of digit d at word d + (d / 32) * 4, so that the
+// 32 bins every lane of a wave sums (16-byte reads, 144 bytes apart) fall on
+// different LDS banks.
+constexpr uint32_t kHistWords = kBins + kBins / 32 * 4;
+__device__ __forceinline__ uint32_t hist_slot(uint32_t digit) { return digit + ((digit >> 1) & ~15u) / 4u; }
+
+// Dynamic LDS of the register path: two histograms (passes alternate, so one
+// barrier per pass is enough), then the listed candidates.  It lies on top of
+// the candidate arrays of the LDS path, which are only filled once this path
+// has given up.
+constexpr size_t kListOff = 2 * (size_t)kHistWords * sizeof(uint32_t);
+constexpr size_t kListWords = kListMax + 8;  // rounded up to whole groups of eight when ranking
+constexpr size_t kLdsBytes = kListOff + 2 * kListWords * sizeof(uint64_t);
+
+struct Shared {
+  uint32_t wave_total[select::kMaxWaves];
+  uint32_t list_count;
+  uint32_t digit, need, count;       // what wave 0 found in the last pass
+  uint64_t cut_key, cut_index;       // the cut, when wave 0 ranked a list
+};
+
+// Inclusive prefix sum over the 64 lanes of a wave, in registers.
+__device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
+  // within rows of 16 lanes: shifts by 1, 2, 4, 8 (lanes without a source add 0)
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false);
+  // lane 15 of a row into the next row (rows 1 and 3), then lane 31 into rows 2 and 3
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);
+  return v;
+}
+
+struct Found { uint32_t digit, need, count; };  // wave-uniform
+
+// One wave, all 64 lanes: the bin that holds the need-th entry (1-based) of
+// `total` counted from the best digit down, the rank left within it (again from
+// the best) and its population.
+__device__ __forceinline__ Found find_bin_wave(const uint32_t* hist, uint32_t need_from_top, uint32_t total,
+                                               uint32_t lane) {
+  const uint32_t need = total - need_from_top + 1u;  // counted from the weakest digit up
+  uint32_t mine = 0;
 #pragma unroll
-      for (int s = 0; s < J; ++s) { cand_key[c * J + s] = (skey_t)E::key(qv[s]); cand_pos[c * J + s] = (pos_t)qp[s]; }
+  for (int i = 0; i < 8; ++i) {
+    const uint4 h = *reinterpret_cast<const uint4*>(&hist[lane * 36u + 4u * i]);
+    mine += h.x + h.y + h.z + h.w;
+  }
+  const uint32_t incl = wave_scan(mine);
+  const uint64_t hit = __ballot(incl - mine < need && need <= incl);
+  const int chunk = __builtin_amdgcn_readfirstlane((int)__ffsll((unsigned long long)hit) - 1);
+  const uint32_t before = (uint32_t)__builtin_amdgcn_readlane((int)(incl - mine), chunk);
+  // the 32 bins of that chunk, one per lane
+  const uint32_t bin = lane < 32u ? hist[(uint32_t)chunk * 36u + lane] : 0u;
+  const uint32_t incl2 = wave_scan(bin);
+  const uint32_t left = need - before;
+  const uint64_t hit2 = __ballot(incl2 - bin < left && left <= incl2);
+  const int at = __builtin_amdgcn_readfirstlane((int)__ffsll((unsigned long long)hit2) - 1);
+  Found f;
+  f.digit = (uint32_t)chunk * 32u + (uint32_t)at;
+  f.count = (uint32_t)__builtin_amdgcn_readlane((int)bin, at);
+  // rank within the bin from its weakest member up, turned round
+  f.need = f.count - (left - (uint32_t)__builtin_amdgcn_readlane((int)(incl2 - bin), at)) + 1u;
+  return f;
+}
+
+}  // namespace regs
+
+// Packed queues of up to 16 entries per lane are held to 64 vector registers
+// (eight waves per SIMD: four 8-wave workgroups per CU); what does not fit is
+// spilled where the pressure peaks, in the rarely taken LDS path.
+template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
+__global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80)))
+__attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_regs_kernel(
+    const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
+    const IndexOut indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t hand_off,
+    uint32_t k0, uint32_t k, int index_bits, int staged) {
+  using raw_t = typename E::raw_t;
+  using skey_t = std::conditional_t<E::key_bits <= 16, uint16_t, typename E::key_t>;
+  using Queue = stream::QueueFor<E, J, V, PACKED, true>;
+  using sel_t = typename Queue::sel_t;
+  // positions in the row fit 32 bits whenever sub-row numbers fit 16 (the candidates fit LDS)
+  using idx_t = std::conditional_t<sizeof(pos_t) == 2, uint32_t, uint64_t>;
+  constexpr int kTileCols = kWave * V;
+  constexpr int NC = V * J;  // candidates per lane
+  constexpr int U = PACKED ? (V * J <= 8 ? 8 : 4) : (J <= 2 ? 8 : 4);
+
+  extern __shared__ __align__(16) unsigned char dyn_lds[];
+  __shared__ select::SharedT<4> sh;  // the LDS path's
+  __shared__ regs::Shared rs;
+  skey_t* cand_key = reinterpret_cast<skey_t*>(dyn_lds);
+  const uint32_t pos_off = (k0 * (uint32_t)sizeof(skey_t) + 15u) & ~15u;
+  pos_t* cand_pos = reinterpret_cast<pos_t*>(dyn_lds + pos_off);
+  unsigned char* hand = dyn_lds + hand_off;
+  uint32_t* hist = reinterpret_cast<uint32_t*>(dyn_lds);  // on top of the candidates: they are parked only after it
+  uint64_t* list_key = reinterpret_cast<uint64_t*>(dyn_lds + regs::kListOff);
+  uint64_t* list_index = list_key + regs::kListWords;
+
+  const uint32_t tid = threadIdx.x, nt = blockDim.x;
+  const uint32_t lane = tid % kWave;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int64_t row = blockIdx.x;
+  const raw_t* xr = x + row * g.row_stride;
+
+  const uint32_t part = wave % split;   // which share of the sub-rows
+  const uint32_t tile = wave / split;   // every tile has its waves: tiles * split == waves
+  const uint32_t p0 = __builtin_amdgcn_readfirstlane((uint32_t)(((uint64_t)g.full_rows * part) / split));
+  const uint32_t p1 = __builtin_amdgcn_readfirstlane((uint32_t)(((uint64_t)g.full_rows * (part + 1)) / split));
+  const bool has_tile = tile < tiles;
+  const int64_t col = (int64_t)tile * kTileCols + lane * V;
+  const bool live = has_tile && col < g.b;
+  const bool mine = live && part == 0;  // this lane ends up holding candidates
+
+  Queue queue;
+  // packed entries: sub-row numbers 0..full_rows at the top of the low half, so
+  // that the bits in which entries differ are the leading ones
+  queue.set_position_shift(sizeof(pos_t) == 2 ? (uint32_t)__builtin_clz(g.full_rows | 1u) - 16u : 0u);
+  bool any_nan = false;
+  if (has_tile) {
+    stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, part == split - 1, queue);
+    any_nan = queue.poisoned();
+  }
+  if (split > 1) {
+    if (has_tile && part > 0)
+      queue.hand_over(hand + (size_t)(tile * (split - 1) + (part - 1)) * Queue::kHandBytes, lane);
+    __syncthreads();
+    if (has_tile && part == 0) {
+      for (uint32_t w = 0; w + 1 < split; ++w)
+        queue.fold_in(hand + (size_t)(tile * (split - 1) + w) * Queue::kHandBytes, lane);
     }
   }
-  // (the select's first pass starts with a barrier, which also publishes the candidates)
+  // Both histograms start at zero.  Waves that shared a tile must first be done
+  // with the hand-over area, which may lie in the same place.
+  if (split > 1) __syncthreads();
+  for (uint32_t i = tid * 4; i < 2 * regs::kHistWords; i += nt * 4)
+    *reinterpret_cast<uint4*>(&hist[i]) = make_uint4(0, 0, 0, 0);
+  if (tid == 0) rs.list_count = 0;
+  const bool nan_row = __syncthreads_or(any_nan);
 
-  auto key_at = [&](uint32_t i) -> key_t { return cand_key[i]; };
-  auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)cand_pos[i] * (uint64_t)g.b + i / J; };
-  const select::Cut<key_t> cut =
-      select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
-
-  raw_t* ov = values + row * (int64_t)k;
-  const int64_t oi = row * (int64_t)k;  // this row's first output slot
-  auto survives = [&](uint32_t i) -> bool {
-    const key_t key = key_at(i);
-    if (key != cut.T) return key > cut.T;
-    return cut.index_cut == ~0ull || index_at(i) <= cut.index_cut;
+  // (keys are taken from the queues where they are used rather than kept: registers)
+  auto key_of = [&](auto e_c) __attribute__((always_inline)) -> sel_t {
+    constexpr int e = decltype(e_c)::value;
+    return queue.template sel_key<e / J, e % J>();
   };
-  // The survivors' values are worked out from their keys; only a key that does
-  // not name one bit pattern (a zero, a NaN) sends its lane to the row.
-  struct Got { int64_t index; raw_t value; };
-  select::compact(
-      sh, k0, k, survives,
-      [&](uint32_t i) {
-        const int64_t index = (int64_t)index_at(i);
-        const key_t key = key_at(i);
-        raw_t value = E::unkey(key);
-        if (!E::key_is_exact(key) && survives(i)) value = xr[index];
-        return Got{index, value};
-      },
-      [&](uint32_t, uint32_t o, const Got& got) {
-        ov[o] = got.value;
-        indices.put(oi + o, got.index);
-      });
+  auto index_of = [&](auto e_c) __attribute__((always_inline)) -> idx_t {
+    constexpr int e = decltype(e_c)::value;
+    return (idx_t)queue.template position<e / J, e % J>() * (idx_t)g.b + (idx_t)(col + e / J);
+  };
+
+  // MSB-first radix passes over sel_key.  After a pass the candidates still in
+  // the race share `prefix` in the bits of `mask`; `need` of those `count` belong
+  // to the result.  The race ends when all of them do (the cut is then the
+  // prefix itself), when they are few enough to be listed and ranked, or, with
+  // no bits left, when they are too many equal keys for that (the LDS path then
+  // cuts them by index).  Pass p counts into histogram p % 2, which the pass
+  // before last left cleared; wave 0 reads it.
+  sel_t prefix = 0, mask = 0;
+  uint32_t need = k, count = k0;
+  enum { kByPrefix, kByList, kGiveUp } how = kGiveUp;
+  if (!nan_row) {
+    int shift = Queue::sel_bits;
+    const int shift_end = queue.sel_constant_bits();
+    for (uint32_t pass = 0;; ++pass) {
+      if (need == count) { how = kByPrefix; break; }
+      if (count <= regs::kListMax) { how = kByList; break; }
+      if (shift <= shift_end) break;
+      const int bits = shift - shift_end < regs::kDigitBits ? shift - shift_end : regs::kDigitBits;
+      shift -= bits;
+      const uint32_t dmask = (1u << bits) - 1u;
+      uint32_t* h = hist + (pass & 1u) * regs::kHistWords;
+      if (mine) {
+        if (pass == 0) {  // every candidate counts
+          ATK_STATIC_FOR(e, NC) {
+            const sel_t key = key_of(std::integral_constant<int, e>{});
+            atomicAdd(&h[regs::hist_slot((uint32_t)(key >> shift) & dmask)], 1u);
+          } ATK_STATIC_END;
+        } else {
+          ATK_STATIC_FOR(e, NC) {
+            const sel_t key = key_of(std::integral_constant<int, e>{});
+            if ((key & mask) == prefix) atomicAdd(&h[regs::hist_slot((uint32_t)(key >> shift) & dmask)], 1u);
+          } ATK_STATIC_END;
+        }
+      }
+      __syncthreads();
+      if (wave == 0) {
+        const regs::Found f = regs::find_bin_wave(h, need, count, lane);
+        if (lane == 0) { rs.digit = f.digit; rs.need = f.need; rs.count = f.count; }
+      }
+      if (pass >= 1) {  // the other histogram, for the pass after this one
+        uint32_t* other = hist + ((pass & 1u) ^ 1u) * regs::kHistWords;
+        for (uint32_t i = tid * 4; i < regs::kHistWords; i += nt * 4)
+          *reinterpret_cast<uint4*>(&other[i]) = make_uint4(0, 0, 0, 0);
+      }
+      __syncthreads();
+      prefix |= (sel_t)rs.digit << shift;
+      mask |= (sel_t)dmask << shift;
+      need = rs.need;
+      count = rs.count;
+    }
+  }
+  if (how == kGiveUp) {
+    // Off the fast path, through the candidate arrays in LDS as in the kernel
+    // above: a NaN in the row (stage 1 again, with exact keys), or more than
+    // kListMax candidates equal to the cut key under sel_key (cut by index).
+    __syncthreads();
+    if (nan_row) {
+      redo_exact_into_lds<E, J>(xr, g, cand_key, cand_pos);
+    } else if (mine) {
+      ATK_STATIC_FOR(e, NC) {
+        cand_key[col * J + e] = (skey_t)queue.template key<e / J, e % J>();
+        cand_pos[col * J + e] = (pos_t)queue.template position<e / J, e % J>();
+      } ATK_STATIC_END;
+    }
+    select_from_lds<E, J>(sh, xr, g, cand_key, cand_pos, k0, k, index_bits, row, values, indices);
+    return;
+  }
+
+  // The cut: a candidate survives when its key is above cut_key, or equal to it
+  // with an index below cut_below.
+  sel_t cut_key;
+  idx_t cut_below;
+  if (how == kByPrefix) {
+    // everything at or above the prefix survives (prefix > 0: something is cut)
+    cut_key = prefix - 1;
+    cut_below = 0;
+  } else {
+    // List the candidates that share the prefix; wave 0 ranks them (lane t takes
+    // entry t and counts the better ones): the need-th best is the cut.  An entry
+    // is one 64-bit word when key and index fit 32 bits each (key above inverted
+    // index: a larger word is a better candidate), else two.  The list is read
+    // eight entries at a time; its last group is filled up with entries that
+    // beat nothing.
+    constexpr bool kOneWord = sizeof(sel_t) == 4 && sizeof(idx_t) == 4;
+    if (tid < 8u) {
+      list_key[count + tid] = 0;
+      list_index[count + tid] = ~0ull;
+    }
+    if (mine) {
+      ATK_STATIC_FOR(e, NC) {
+        const sel_t key = key_of(std::integral_constant<int, e>{});
+        if ((key & mask) == prefix) {
+          const uint32_t slot = atomicAdd(&rs.list_count, 1u);
+          const idx_t index = index_of(std::integral_constant<int, e>{});
+          if constexpr (kOneWord) {
+            list_key[slot] = ((uint64_t)key << 32) | (uint64_t)(0xffffffffu - (uint32_t)index);
+          } else {
+            list_key[slot] = (uint64_t)key;
+            list_index[slot] = (uint64_t)index;
+          }
+        }
+      } ATK_STATIC_END;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const uint32_t t = lane < count ? lane : 0u;
+      const uint64_t my_key = list_key[t];
+      const uint64_t my_index = kOneWord ? 0ull : list_index[t];
+      uint32_t better = 0;
+      for (uint32_t m = 0; m < count; m += 8) {
+        uint64_t key[8], index[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { key[u] = list_key[m + u]; index[u] = kOneWord ? 0ull : list_index[m + u]; }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          better += (key[u] > my_key || (!kOneWord && key[u] == my_key && index[u] < my_index)) ? 1u : 0u;
+      }
+      if (lane < count && better + 1 == need) {  // one lane
+        rs.cut_key = my_key;
+        rs.cut_index = my_index;
+      }
+    }
+    __syncthreads();
+    if constexpr (kOneWord) {
+      cut_key = (sel_t)(rs.cut_key >> 32);
+      cut_below = (idx_t)(0xffffffffu - (uint32_t)rs.cut_key) + 1u;
+    } else {
+      cut_key = (sel_t)rs.cut_key;
+      cut_below = (idx_t)rs.cut_index + 1u;
+    }
+  }
+
+  // survivors, one bit per candidate of this lane
+  if (mine) queue.fix_zeros(xr, g.b, col);
+  uint32_t selected = 0;
+  ATK_STATIC_FOR(e, NC) {
+    const sel_t key = key_of(std::integral_constant<int, e>{});
+    bool sel = key > cut_key;
+    if (key == cut_key) sel = index_of(std::integral_constant<int, e>{}) < cut_below;
+    selected |= (mine && sel) ? (1u << e) : 0u;
+  } ATK_STATIC_END;
+  const uint32_t kept = (uint32_t)__popc(selected);
+  const uint32_t incl = regs::wave_scan(kept);
+  if (lane == kWave - 1) rs.wave_total[wave] = incl;
+  __syncthreads();
+  uint32_t o = incl - kept;
+  for (uint32_t w = 0; w < wave; ++w) o += rs.wave_total[w];
+  raw_t* ov = values + row * (int64_t)k;
+  const int64_t oi = row * (int64_t)k;
+  if constexpr (sizeof(idx_t) == 4 && sizeof(raw_t) <= 4) {
+    if (staged != 0) {
+      // Survivors go to LDS first (element and index, eight bytes, at their output
+      // slot), so that the row's results leave in whole-wave stores.  The area
+      // lies on top of the histograms and the list, which nobody reads any more
+      // (the barrier above).
+      uint2* stage = reinterpret_cast<uint2*>(dyn_lds);
+      ATK_STATIC_FOR(e, NC) {
+        if ((selected >> e) & 1u) {
+          if (o < k)
+            stage[o] = make_uint2((uint32_t)queue.template raw<e / J, e % J>(),
+                                  (uint32_t)index_of(std::integral_constant<int, e>{}));
+          ++o;
+        }
+      } ATK_STATIC_END;
+      __syncthreads();
+      if (staged == 2) {  // four results per thread: k is a multiple of four and the outputs are 16-byte aligned
+        for (uint32_t at = tid * 4; at < k; at += nt * 4) {
+          const uint4 e01 = *reinterpret_cast<const uint4*>(&stage[at]);
+          const uint4 e23 = *reinterpret_cast<const uint4*>(&stage[at + 2]);
+          stream::Pack<raw_t, 4> pv;
+          pv.e[0] = (raw_t)e01.x; pv.e[1] = (raw_t)e01.z; pv.e[2] = (raw_t)e23.x; pv.e[3] = (raw_t)e23.z;
+          *reinterpret_cast<stream::Pack<raw_t, 4>*>(ov + at) = pv;
+          if (indices.narrow) {
+            stream::Pack<int32_t, 4> pi;
+            pi.e[0] = (int32_t)e01.y; pi.e[1] = (int32_t)e01.w; pi.e[2] = (int32_t)e23.y; pi.e[3] = (int32_t)e23.w;
+            *reinterpret_cast<stream::Pack<int32_t, 4>*>(static_cast<int32_t*>(indices.base) + oi + at) = pi;
+          } else {
+            int64_t* out = static_cast<int64_t*>(indices.base) + oi + at;
+            stream::Pack<int64_t, 2> lo, hi;
+            lo.e[0] = (int64_t)e01.y; lo.e[1] = (int64_t)e01.w; hi.e[0] = (int64_t)e23.y; hi.e[1] = (int64_t)e23.w;
+            reinterpret_cast<stream::Pack<int64_t, 2>*>(out)[0] = lo;
+            reinterpret_cast<stream::Pack<int64_t, 2>*>(out)[1] = hi;
+          }
+        }
+      } else {
+        for (uint32_t at = tid; at < k; at += nt) {
+          const uint2 got = stage[at];
+          ov[at] = (raw_t)got.x;
+          indices.put(oi + at, (int64_t)got.y);
+        }
+      }
+      return;
+    }
+  }
+  ATK_STATIC_FOR(e, NC) {
+    if ((selected >> e) & 1u) {
+      if (o < k) {
+        ov[o] = queue.template raw<e / J, e % J>();
+        indices.put(oi + o, (int64_t)index_of(std::integral_constant<int, e>{}));
+      }
+      ++o;
+    }
+  } ATK_STATIC_END;
 }
 
 // ---------------------------------------------------------------------------
@@ -164,6 +557,8 @@ struct Plan {
   int index_bits;
   uint32_t hand_off;    // byte offset of the hand-over area in dynamic LDS (0: on top of the candidates)
   size_t lds_bytes;     // dynamic LDS
+  bool in_registers;    // all tiles are scanned at once: the candidates stay in registers through stage 2
+  bool staged;          // in_registers: the survivors are gathered in LDS and leave in whole-wave stores
 };
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned);

@@ -9,6 +9,20 @@ namespace fused {
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
 static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                          uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
+  if (pl.in_registers) {
+    auto kern = fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED>;
+    if (pl.lds_bytes > 48 * 1024) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)pl.lds_bytes) != hipSuccess)
+        return ATK_ERR_LAUNCH;
+    }
+    // staged results leave four per thread when the outputs allow 16-byte stores
+    const bool wide = k % 4 == 0 && (uintptr_t)values % 16 == 0 && (uintptr_t)indices.base % 16 == 0;
+    const int staged = pl.staged ? (wide ? 2 : 1) : 0;
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(kWave * pl.waves), pl.lds_bytes, stream, x, values,
+                       indices, g, pl.tiles, pl.split, pl.hand_off, k0, k, pl.index_bits, staged);
+    return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+  }
   auto kern = fused_row_kernel<E, J, V, MAXW, pos_t, PACKED>;
   if (pl.lds_bytes > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

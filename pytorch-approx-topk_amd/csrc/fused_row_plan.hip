@@ -99,6 +99,13 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   const bool one_round = pl.tiles * split <= kMaxWaves;
   pl.hand_off = (split > 1 && !one_round) ? (uint32_t)cand_bytes : 0u;
   pl.lds_bytes = lds_need(split);
+  // every tile has its waves: stage 2 runs on the candidates where they are, in
+  // registers, and needs the histogram's room in LDS
+  pl.in_registers = one_round;
+  if (pl.in_registers && pl.lds_bytes < regs::kLdsBytes) pl.lds_bytes = regs::kLdsBytes;
+  // survivors staged in LDS, eight bytes each (element, 32-bit index), when that fits
+  pl.staged = pl.in_registers && pl.pos16 && es <= 4 && (size_t)k * 8 <= kLdsBudget;
+  if (pl.staged && pl.lds_bytes < (size_t)k * 8) pl.lds_bytes = (size_t)k * 8;
   pl.ok = true;
   return pl;
 }

@@ -199,6 +199,9 @@ template <typename E, int J, int V> struct CmpQueue {
   uint64_t nan_mask;  // lanes that loaded a NaN; wave-uniform
 
   __device__ __forceinline__ void reset() { nan_mask = 0; }
+  __device__ __forceinline__ void set_position_shift(uint32_t) {}
+  // low bits of sel_key that are the same in every entry
+  __device__ __forceinline__ int sel_constant_bits() const { return 0; }
 
   // FILLED: how many entries every column already holds (the first J sub-rows fill the queues)
   template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
@@ -249,6 +252,12 @@ template <typename E, int J, int V> struct CmpQueue {
   __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t) {}
   // exact order key of an entry (the queues are not poisoned)
   template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return E::key(C::to_raw(q[VI][SI])); }
+  // A key cheap to get from an entry whose order is the selection order as far
+  // as it goes: entries with different sel_key rank by it, entries with equal
+  // sel_key by their index (lower first).
+  using sel_t = typename E::key_t;
+  static constexpr int sel_bits = E::key_bits;
+  template <int VI, int SI> __device__ __forceinline__ sel_t sel_key() const { return key<VI, SI>(); }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const { return C::to_raw(q[VI][SI]); }
   template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return pos[VI][SI]; }
 };
@@ -323,7 +332,7 @@ template <int J> __device__ __forceinline__ void insert_word(uint32_t (&col)[J],
   col[J - 1] = col[J - 1] > word ? col[J - 1] : word;
 }
 
-template <typename E, int J, int V> struct PackedQueue {
+template <typename E, int J, int V, bool SHIFTED = false> struct PackedQueue {
   using raw_t = typename E::raw_t;
   using K = PackedKey<E>;
   static_assert(sizeof(raw_t) == 2 && (V % 2 == 0 || V == 1), "packed queues hold 16-bit elements");
@@ -332,7 +341,28 @@ template <typename E, int J, int V> struct PackedQueue {
   uint32_t q[V][J];
   uint32_t screen;     // NaN screen, two halves
   uint32_t neg_zeros;  // bit v*J+s: entry (v, s) is a -0.0 (set by fix_zeros)
+  // The low half of an entry holds 0xffff - sub-row, or, SHIFTED, that value
+  // shifted left by `pshift` within the half: when sub-row numbers need only
+  // 16 - pshift bits, this puts every bit in which the entries of a run differ
+  // at the top of the word (wave-uniform; SHIFTED = false keeps no such member).
+  struct None {};
+  [[no_unique_address]] std::conditional_t<SHIFTED, uint32_t, None> pshift;
 
+  __device__ __forceinline__ void set_position_shift(uint32_t shift) {
+    if constexpr (SHIFTED) pshift = shift;
+  }
+  __device__ __forceinline__ int sel_constant_bits() const {
+    if constexpr (SHIFTED) return (int)pshift;
+    return 0;
+  }
+  __device__ __forceinline__ uint32_t low_half(uint32_t p) const {
+    if constexpr (SHIFTED) return ((0xffffu - p) << pshift) & 0xffffu;
+    return 0xffffu - p;
+  }
+  __device__ __forceinline__ uint32_t sub_row(uint32_t word) const {
+    if constexpr (SHIFTED) return (0xffffu >> pshift) - ((word & 0xffffu) >> pshift);
+    return 0xffffu - (word & 0xffffu);
+  }
   __device__ __forceinline__ void reset() {
     ATK_STATIC_FOR(e, V * J) { q[e / J][e % J] = 0; } ATK_STATIC_END;
     screen = 0;
@@ -340,7 +370,7 @@ template <typename E, int J, int V> struct PackedQueue {
   }
   __device__ static __forceinline__ void insert(uint32_t (&col)[J], uint32_t word) { insert_word<J>(col, word); }
   template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
-    const uint32_t pinv = 0xffffu - p;
+    const uint32_t pinv = low_half(p);
     if constexpr (V == 1) {
       const uint32_t keys = K::keys2(pk.e[0], screen);
       insert(q[0], (keys << 16) | pinv);
@@ -359,7 +389,7 @@ template <typename E, int J, int V> struct PackedQueue {
     uint32_t scr = screen;
     const uint32_t keys = K::keys2((uint32_t)raw, scr);  // the empty high half screens as +0
     if (valid) screen = scr;
-    insert(q[VI], valid ? ((keys << 16) | (0xffffu - p)) : 0u);
+    insert(q[VI], valid ? ((keys << 16) | low_half(p)) : 0u);
   }
   __device__ __forceinline__ bool poisoned() const { return __ballot(K::special(screen)) != 0; }
 
@@ -381,7 +411,7 @@ template <typename E, int J, int V> struct PackedQueue {
       ATK_STATIC_FOR(e, V * J) {
         const uint32_t word = q[e / J][e % J];
         if ((word >> 16) == K::kZeroKey) {
-          const uint32_t p = 0xffffu - (word & 0xffffu);
+          const uint32_t p = sub_row(word);
           if (xr[(int64_t)p * b + col + e / J] == (raw_t)0x8000u) neg_zeros |= 1u << e;
         }
       } ATK_STATIC_END;
@@ -389,12 +419,17 @@ template <typename E, int J, int V> struct PackedQueue {
   }
   // exact order key of an entry (the queues are not poisoned)
   template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return K::exact(q[VI][SI] >> 16); }
+  // the entry's word as it is: packed key, then lower sub-row first -- the
+  // selection order up to the column, which is what the index decides last
+  using sel_t = uint32_t;
+  static constexpr int sel_bits = 32;
+  template <int VI, int SI> __device__ __forceinline__ sel_t sel_key() const { return q[VI][SI]; }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
     const raw_t r = K::unkey(q[VI][SI] >> 16);
     if constexpr (K::zero_is_ambiguous) return (neg_zeros >> (VI * J + SI)) & 1u ? (raw_t)0x8000u : r;
     return r;
   }
-  template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return 0xffffu - (q[VI][SI] & 0xffffu); }
+  template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return sub_row(q[VI][SI]); }
 };
 
 // The same for 8-bit element types and rows of fewer than 2^24 - 1 sub-rows:
@@ -418,6 +453,8 @@ template <typename E, int J, int V> struct ByteQueue {
   __device__ __forceinline__ void reset() {
     ATK_STATIC_FOR(e, V * J) { q[e / J][e % J] = 0; } ATK_STATIC_END;
   }
+  __device__ __forceinline__ void set_position_shift(uint32_t) {}
+  __device__ __forceinline__ int sel_constant_bits() const { return 0; }
   __device__ static __forceinline__ void insert(uint32_t (&col)[J], uint32_t word) { insert_word<J>(col, word); }
   template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
     const uint32_t pinv = 0xffffffu - p;
@@ -452,16 +489,19 @@ template <typename E, int J, int V> struct ByteQueue {
   }
   __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t) {}
   template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return q[VI][SI] >> 24; }
+  using sel_t = uint32_t;
+  static constexpr int sel_bits = 32;
+  template <int VI, int SI> __device__ __forceinline__ sel_t sel_key() const { return q[VI][SI]; }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
     return (raw_t)((q[VI][SI] >> 24) ^ (K::kFlip & 0xffu));
   }
   template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return 0xffffffu - (q[VI][SI] & 0xffffffu); }
 };
 
-template <typename E, int J, int V, bool PACKED>
+template <typename E, int J, int V, bool PACKED, bool SHIFTED = false>
 using QueueFor = std::conditional_t<
     !PACKED, CmpQueue<E, J, V>,
-    std::conditional_t<sizeof(typename E::raw_t) == 1, ByteQueue<E, J, V>, PackedQueue<E, J, V>>>;
+    std::conditional_t<sizeof(typename E::raw_t) == 1, ByteQueue<E, J, V>, PackedQueue<E, J, V, SHIFTED>>>;
 
 // Shape of one launch; passed to the kernels by value.  With few buckets the
 // planner folds the row: `fold` consecutive sub-rows of the true [L][b] matrix
