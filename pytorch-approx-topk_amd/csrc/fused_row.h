@@ -469,14 +469,13 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
     }
   }
 
-  // survivors, one bit per candidate of this lane
-  if (mine) queue.fix_zeros(xr, g.b, col);
-  uint32_t selected = 0;
+  // survivors among this lane's candidates
+  uint32_t selected = 0;  // bit e: candidate e survives
   ATK_STATIC_FOR(e, NC) {
     const sel_t key = key_of(std::integral_constant<int, e>{});
-    bool sel = key > cut_key;
-    if (key == cut_key) sel = index_of(std::integral_constant<int, e>{}) < cut_below;
-    selected |= (mine && sel) ? (1u << e) : 0u;
+    bool s = key > cut_key;
+    if (key == cut_key) s = index_of(std::integral_constant<int, e>{}) < cut_below;
+    selected |= (mine && s) ? (1u << e) : 0u;
   } ATK_STATIC_END;
   const uint32_t kept = (uint32_t)__popc(selected);
   const uint32_t incl = regs::wave_scan(kept);
@@ -488,49 +487,62 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
   const int64_t oi = row * (int64_t)k;
   if constexpr (sizeof(idx_t) == 4 && sizeof(raw_t) <= 4) {
     if (staged != 0) {
-      // Survivors go to LDS first (element and index, eight bytes, at their output
-      // slot), so that the row's results leave in whole-wave stores.  The area
+      // Survivors go to LDS first, as their queue entries and columns at their
+      // output slots (eight bytes each; exactly k of them), and the threads that
+      // carry the row's results out in whole-wave stores turn them into elements
+      // and indices: a quarter as many conversions as candidates.  The area
       // lies on top of the histograms and the list, which nobody reads any more
       // (the barrier above).
       uint2* stage = reinterpret_cast<uint2*>(dyn_lds);
       ATK_STATIC_FOR(e, NC) {
-        if ((selected >> e) & 1u) {
-          if (o < k)
-            stage[o] = make_uint2((uint32_t)queue.template raw<e / J, e % J>(),
-                                  (uint32_t)index_of(std::integral_constant<int, e>{}));
-          ++o;
-        }
+        if ((selected >> e) & 1u) stage[o] = queue.template staged<e / J, e % J>((uint32_t)col + e / J);
+        o += (selected >> e) & 1u;
       } ATK_STATIC_END;
       __syncthreads();
+      auto result = [&](uint2 w, raw_t& value) __attribute__((always_inline)) -> uint32_t {
+        const typename Queue::Unstaged u = queue.unstage(w);
+        const uint32_t index = u.sub_row * (uint32_t)g.b + u.column;
+        value = u.raw;
+        if (u.reread) value = xr[index];  // a zero: its sign is in the row
+        return index;
+      };
       if (staged == 2) {  // four results per thread: k is a multiple of four and the outputs are 16-byte aligned
         for (uint32_t at = tid * 4; at < k; at += nt * 4) {
           const uint4 e01 = *reinterpret_cast<const uint4*>(&stage[at]);
           const uint4 e23 = *reinterpret_cast<const uint4*>(&stage[at + 2]);
           stream::Pack<raw_t, 4> pv;
-          pv.e[0] = (raw_t)e01.x; pv.e[1] = (raw_t)e01.z; pv.e[2] = (raw_t)e23.x; pv.e[3] = (raw_t)e23.z;
+          uint32_t index[4];
+          index[0] = result(make_uint2(e01.x, e01.y), pv.e[0]);
+          index[1] = result(make_uint2(e01.z, e01.w), pv.e[1]);
+          index[2] = result(make_uint2(e23.x, e23.y), pv.e[2]);
+          index[3] = result(make_uint2(e23.z, e23.w), pv.e[3]);
           *reinterpret_cast<stream::Pack<raw_t, 4>*>(ov + at) = pv;
           if (indices.narrow) {
             stream::Pack<int32_t, 4> pi;
-            pi.e[0] = (int32_t)e01.y; pi.e[1] = (int32_t)e01.w; pi.e[2] = (int32_t)e23.y; pi.e[3] = (int32_t)e23.w;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) pi.e[u] = (int32_t)index[u];
             *reinterpret_cast<stream::Pack<int32_t, 4>*>(static_cast<int32_t*>(indices.base) + oi + at) = pi;
           } else {
             int64_t* out = static_cast<int64_t*>(indices.base) + oi + at;
             stream::Pack<int64_t, 2> lo, hi;
-            lo.e[0] = (int64_t)e01.y; lo.e[1] = (int64_t)e01.w; hi.e[0] = (int64_t)e23.y; hi.e[1] = (int64_t)e23.w;
+            lo.e[0] = (int64_t)index[0]; lo.e[1] = (int64_t)index[1];
+            hi.e[0] = (int64_t)index[2]; hi.e[1] = (int64_t)index[3];
             reinterpret_cast<stream::Pack<int64_t, 2>*>(out)[0] = lo;
             reinterpret_cast<stream::Pack<int64_t, 2>*>(out)[1] = hi;
           }
         }
       } else {
         for (uint32_t at = tid; at < k; at += nt) {
-          const uint2 got = stage[at];
-          ov[at] = (raw_t)got.x;
-          indices.put(oi + at, (int64_t)got.y);
+          raw_t value;
+          const uint32_t index = result(stage[at], value);
+          ov[at] = value;
+          indices.put(oi + at, (int64_t)index);
         }
       }
       return;
     }
   }
+  if (mine) queue.fix_zeros(xr, g.b, col);
   ATK_STATIC_FOR(e, NC) {
     if ((selected >> e) & 1u) {
       if (o < k) {

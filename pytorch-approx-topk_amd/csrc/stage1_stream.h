@@ -258,6 +258,16 @@ template <typename E, int J, int V> struct CmpQueue {
   using sel_t = typename E::key_t;
   static constexpr int sel_bits = E::key_bits;
   template <int VI, int SI> __device__ __forceinline__ sel_t sel_key() const { return key<VI, SI>(); }
+  // An entry as two 32-bit words for a hand-over that is undone elsewhere
+  // (elements of at most four bytes, sub-row numbers and columns below 65536):
+  // what `unstage` needs to give back the element and where it came from.
+  template <int VI, int SI> __device__ __forceinline__ uint2 staged(uint32_t column) const {
+    return make_uint2((uint32_t)C::to_raw(q[VI][SI]), (pos[VI][SI] << 16) | column);
+  }
+  struct Unstaged { raw_t raw; uint32_t sub_row, column; bool reread; };  // reread: take the element from the row
+  __device__ __forceinline__ Unstaged unstage(uint2 w) const {
+    return Unstaged{(raw_t)w.x, w.y >> 16, w.y & 0xffffu, false};
+  }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const { return C::to_raw(q[VI][SI]); }
   template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return pos[VI][SI]; }
 };
@@ -424,6 +434,15 @@ template <typename E, int J, int V, bool SHIFTED = false> struct PackedQueue {
   using sel_t = uint32_t;
   static constexpr int sel_bits = 32;
   template <int VI, int SI> __device__ __forceinline__ sel_t sel_key() const { return q[VI][SI]; }
+  template <int VI, int SI> __device__ __forceinline__ uint2 staged(uint32_t column) const {
+    return make_uint2(q[VI][SI], column);
+  }
+  struct Unstaged { raw_t raw; uint32_t sub_row, column; bool reread; };
+  __device__ __forceinline__ Unstaged unstage(uint2 w) const {
+    bool zero = false;
+    if constexpr (K::zero_is_ambiguous) zero = (w.x >> 16) == K::kZeroKey;
+    return Unstaged{K::unkey(w.x >> 16), sub_row(w.x), w.y, zero};
+  }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
     const raw_t r = K::unkey(q[VI][SI] >> 16);
     if constexpr (K::zero_is_ambiguous) return (neg_zeros >> (VI * J + SI)) & 1u ? (raw_t)0x8000u : r;
@@ -492,6 +511,13 @@ template <typename E, int J, int V> struct ByteQueue {
   using sel_t = uint32_t;
   static constexpr int sel_bits = 32;
   template <int VI, int SI> __device__ __forceinline__ sel_t sel_key() const { return q[VI][SI]; }
+  template <int VI, int SI> __device__ __forceinline__ uint2 staged(uint32_t column) const {
+    return make_uint2(q[VI][SI], column);
+  }
+  struct Unstaged { raw_t raw; uint32_t sub_row, column; bool reread; };
+  __device__ __forceinline__ Unstaged unstage(uint2 w) const {
+    return Unstaged{(raw_t)((w.x >> 24) ^ (K::kFlip & 0xffu)), 0xffffffu - (w.x & 0xffffffu), w.y, false};
+  }
   template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
     return (raw_t)((q[VI][SI] >> 24) ^ (K::kFlip & 0xffu));
   }
