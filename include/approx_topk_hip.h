@@ -151,6 +151,18 @@ int atk_topk_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride,
                  void* ws, size_t ws_bytes, atk_stream_t stream);
 
 /*
+ * Diagnostics: which kernels atk_topk (atk_stage1 when k == k0) would enqueue
+ * for these arguments, as text ("name<parameters> grid=... block=...", several
+ * kernels joined by " + "), truncated to text_bytes - 1 characters.  Enqueues
+ * nothing.  No counterpart in the reference, whose dispatch is one templated
+ * launch (cu:306-375); here the planner picks among several kernels, and a
+ * benchmark record should say which one it timed.
+ */
+int atk_describe(const void* x, int64_t rows, int64_t n, int64_t row_stride,
+                 int64_t k0, int j, int64_t k, int layout, int dtype,
+                 const void* values, const void* indices, char* text, size_t text_bytes);
+
+/*
  * atk_topk without a workspace argument and without any allocation.  No
  * counterpart in the reference: it is for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that

@@ -45,6 +45,9 @@ _SIGNATURES = {
                                                                            ctypes.c_int, ctypes.c_int]
                  + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
                     ctypes.c_void_p]),
+    "atk_describe": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4
+                     + [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]
+                     + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
     "atk_topk_noalloc": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_int64] * 4
                          + [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]
                          + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
@@ -153,25 +156,51 @@ def rows_view(xs: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
     return xs, rows, n, step
 
 
+# Per-call constants of a contiguous input, keyed by everything they depend on:
+# (rows, n, dtype code, output shape, bound entry point).  One dictionary lookup
+# replaces the shape arithmetic on the way to the native call.
+_CALLS: dict = {}
+
+
+def _call_constants(xs: torch.Tensor, k_out: int, two_stage: bool, index_dtype: torch.dtype):
+    key = (xs.shape, xs.dtype, k_out, two_stage, index_dtype)
+    hit = _CALLS.get(key)
+    if hit is None:
+        L = lib()
+        n = xs.shape[-1]
+        rows = xs.numel() // n if n else 0
+        narrow = index_dtype != torch.int64
+        if two_stage:
+            entry = L.atk_topk_i32 if narrow else L.atk_topk
+        else:
+            entry = L.atk_stage1_i32 if narrow else L.atk_stage1
+        hit = (rows, n, dtype_code(xs.dtype), tuple(xs.shape[:-1]) + (k_out,), entry)
+        if len(_CALLS) < 4096:
+            _CALLS[key] = hit
+    return hit
+
+
 def stage1(xs: torch.Tensor, k0: int, j: int, layout: int,
            index_dtype: torch.dtype = torch.int64) -> tuple[torch.Tensor, torch.Tensor]:
     """Per-bucket top-j along the last dim: (values[..., k0], indices[..., k0]).
 
     ``index_dtype``: torch.int64 (the operator's contract) or torch.int32."""
     require_gpu(xs)
-    L = lib()
-    xs, rows, n, step = rows_view(xs)
-    code = dtype_code(xs.dtype)
-    shape = list(xs.shape[:-1]) + [k0]
-    values = torch.empty(shape, dtype=xs.dtype, device=xs.device)
-    indices = torch.empty(shape, dtype=index_dtype, device=xs.device)
-    entry = L.atk_stage1 if index_dtype == torch.int64 else L.atk_stage1_i32
-    with _on_device(xs.device):
+    step = None
+    if not xs.is_contiguous():
+        xs, _, _, step = rows_view(xs)
+    rows, n, code, shape, entry = _call_constants(xs, k0, False, index_dtype)
+    device = xs.device
+    values = torch.empty(shape, dtype=xs.dtype, device=device)
+    indices = torch.empty(shape, dtype=index_dtype, device=device)
+    with _on_device(device):
         need = _stage1_workspace(rows, n, k0, j, layout, code)
-        ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
-        check(entry(xs.data_ptr(), rows, n, step, k0, j, layout, code,
-                           values.data_ptr(), indices.data_ptr(),
-                           ws.data_ptr() if ws is not None else None, need, _stream(xs.device)))
+        ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
+        status = entry(xs.data_ptr(), rows, n, n if step is None else step, k0, j, layout, code,
+                       values.data_ptr(), indices.data_ptr(),
+                       ws.data_ptr() if ws is not None else None, need, _stream(device))
+    if status != 0:
+        check(status)
     return values, indices
 
 
@@ -200,17 +229,30 @@ def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int,
          index_dtype: torch.dtype = torch.int64) -> tuple[torch.Tensor, torch.Tensor]:
     """Stage 1 (k0 candidates) and stage 2 (k survivors) along the last dim."""
     require_gpu(xs)
-    L = lib()
-    xs, rows, n, step = rows_view(xs)
-    code = dtype_code(xs.dtype)
-    shape = list(xs.shape[:-1]) + [k]
-    values = torch.empty(shape, dtype=xs.dtype, device=xs.device)
-    indices = torch.empty(shape, dtype=index_dtype, device=xs.device)
-    entry = L.atk_topk if index_dtype == torch.int64 else L.atk_topk_i32
-    with _on_device(xs.device):
-        need = _topk_workspace(xs.data_ptr() % 16, rows, n, step, k0, j, k, layout, code)
-        ws = torch.empty(need, dtype=torch.uint8, device=xs.device) if need else None
-        check(entry(xs.data_ptr(), rows, n, step, k0, j, k, layout, code,
-                         values.data_ptr(), indices.data_ptr(),
-                         ws.data_ptr() if ws is not None else None, need, _stream(xs.device)))
+    step = None
+    if not xs.is_contiguous():
+        xs, _, _, step = rows_view(xs)
+    rows, n, code, shape, entry = _call_constants(xs, k, True, index_dtype)
+    device = xs.device
+    values = torch.empty(shape, dtype=xs.dtype, device=device)
+    indices = torch.empty(shape, dtype=index_dtype, device=device)
+    with _on_device(device):
+        pitch = n if step is None else step
+        need = _topk_workspace(xs.data_ptr() % 16, rows, n, pitch, k0, j, k, layout, code)
+        ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
+        status = entry(xs.data_ptr(), rows, n, pitch, k0, j, k, layout, code,
+                       values.data_ptr(), indices.data_ptr(),
+                       ws.data_ptr() if ws is not None else None, need, _stream(device))
+    if status != 0:
+        check(status)
     return values, indices
+
+
+def describe(xs: torch.Tensor, k0: int, j: int, k: int, layout: int = INTERLEAVED) -> str:
+    """The kernels a call on `xs` (top-k along the last dim) would launch, as text."""
+    xs, rows, n, step = rows_view(xs)
+    buf = ctypes.create_string_buffer(1024)
+    # outputs of torch.empty are at least 256-byte aligned: any such address stands for them
+    check(lib().atk_describe(xs.data_ptr() if xs.numel() else 4096, rows, n, step, k0, j, k, layout,
+                             dtype_code(xs.dtype), 4096, 4096, buf, len(buf)))
+    return buf.value.decode()

@@ -86,11 +86,15 @@ def _topk(
     if k0 > n:
         raise RuntimeError("topk: k must not be larger than topk size")
     _native.require_gpu(xs)
+    layout = _native.INTERLEAVED if interleaved else _native.BALANCED
+    if dim == last and n != 0 and xs.ndim and xs.numel():  # the common case, straight through
+        if k_mult == 1:
+            return _native.stage1(xs, k0, j, layout, index_dtype)
+        return _native.topk(xs, k0, j, k, layout, index_dtype)
     if xs.numel() == 0:
         values, indices = _empty_result(xs, k, dim)
         return values, indices.to(index_dtype)
 
-    layout = _native.INTERLEAVED if interleaved else _native.BALANCED
     rows = xs if xs.ndim else xs.reshape(1)
     moved = dim != last and xs.ndim > 1
     if moved:

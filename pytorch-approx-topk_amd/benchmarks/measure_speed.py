@@ -5,7 +5,10 @@ Covers the grid of the reference's benchmarks/measure_speed.py:264-327
 (n in 2^12..2^16, batch in {128, 32}, k in {64, n/8}, fp32; torch.topk, the
 approximate top-k at j in {1, 2, 4}, and the torch-level bucketed arg-max), once
 with plain launches and once with the inner loop captured in a HIP graph, timed
-with events as benchmarks/measure_speed.py:98-146 does.  Every line carries the
+with events as benchmarks/measure_speed.py:98-146 does, a device-side spin queued
+ahead of every timed repetition included (:141): the host gets ahead of the GPU
+while the spin runs, so that the events bracket the kernels and not the time the
+host needs to enqueue them.  Every line carries the
 per-call durations in seconds; input bandwidth is dtype_bytes * n * batch / mean
 (benchmarks/plot_bandwidth.py:41-45).
 
@@ -32,9 +35,18 @@ def exact_topk(xs, k, dim):
     return torch.topk(xs, k, dim, sorted=False)
 
 
+# Device clock ticks the GPU spins before each timed repetition (torch.cuda._sleep; the reference
+# spins 10 M cycles, several milliseconds).  Long enough for the host to enqueue `n_inner` calls
+# and the closing event behind it: ~100 us cover a few un-graphed calls or one graph launch.
+HIDE_LAUNCH_CYCLES = 200_000
+
+
 def time_calls(call: Callable[[int], Any], refresh: Callable[[], None], n_outer: int, n_inner: int,
-               graph: bool, n_warmup: int = 16) -> list[float]:
-    """Seconds per call for `n_outer` timed repetitions of `n_inner` calls each."""
+               graph: bool, n_warmup: int = 16, hide_launch_cycles: int = HIDE_LAUNCH_CYCLES) -> list[float]:
+    """Seconds per call for `n_outer` timed repetitions of `n_inner` calls each.
+
+    `hide_launch_cycles` > 0 queues a device-side spin of that many clock ticks ahead of the
+    opening event of every repetition (benchmarks/measure_speed.py:135-146 in the reference)."""
     def inner():
         return [call(i) for i in range(n_inner)]
 
@@ -57,6 +69,8 @@ def time_calls(call: Callable[[int], Any], refresh: Callable[[], None], n_outer:
               for _ in range(n_outer)]
     for start, stop in events:
         refresh()
+        if hide_launch_cycles > 0:
+            torch.cuda._sleep(hide_launch_cycles)
         start.record()
         run()
         stop.record()

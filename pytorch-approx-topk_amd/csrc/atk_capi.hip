@@ -1,6 +1,7 @@
 // extern "C" entry points of libapprox_topk_hip.so: argument checks and the
 // choice of kernel.  Everything here runs on the host and only enqueues work.
 #include <mutex>
+#include <string>
 
 #include "atk_device.h"
 #include "atk_launch.h"
@@ -253,6 +254,37 @@ int atk_topk_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride, int
                  size_t ws_bytes, atk_stream_t stream) {
   return do_topk(x, rows, n, row_stride, k0, j, k, layout, dtype, values, atk::IndexOut{indices, 1}, ws,
                  ws_bytes, (hipStream_t)stream);
+}
+
+int atk_describe(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
+                 int layout, int dtype, const void* values, const void* indices, char* text,
+                 size_t text_bytes) {
+  if (k < 0 || k > k0) return ATK_ERR_K;
+  const int rc = check_stage1(x, rows, n, row_stride, k0, j, layout, dtype, values, indices);
+  if (rc != ATK_OK) return rc;
+  if (!text || text_bytes == 0) return ATK_ERR_ARG;
+  std::string out;
+  if (rows != 0 && k != 0) {
+    bool fused = false;
+    if (k < k0) fused = atk::describe_fused_row(x, rows, n, row_stride, k0, j, k, layout, dtype, out);
+    if (!fused) {
+      // the candidates of a two-stage call are written to the (aligned) workspace
+      const void* v1 = k < k0 ? nullptr : values;
+      const void* i1 = k < k0 ? nullptr : indices;
+      if (!atk::describe_stage1_stream(x, rows, n, row_stride, k0, j, layout, dtype, v1, i1, out) &&
+          !atk::describe_stage1_contig(x, rows, n, row_stride, k0, j, layout, dtype, out))
+        atk::describe_stage1_lane_per_bucket(rows, k0, j, dtype, out);
+      if (k < k0) {
+        out += " + ";
+        if (!atk::describe_multi_select(rows, k0, k, index_bound_of(n, k0, layout), dtype, out))
+          atk::describe_select(rows, k0, k, dtype, true, out);
+      }
+    }
+  }
+  const size_t len = out.size() < text_bytes - 1 ? out.size() : text_bytes - 1;
+  __builtin_memcpy(text, out.data(), len);
+  text[len] = 0;
+  return ATK_OK;
 }
 
 int atk_topk_noalloc(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,

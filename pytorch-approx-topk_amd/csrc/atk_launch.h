@@ -6,6 +6,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <string>
+
 #include "atk_device.h"
 
 namespace atk {
@@ -61,5 +63,20 @@ size_t multi_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dty
 int launch_multi_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
                         int64_t k, int64_t index_bound, int dtype, void* values, IndexOut indices, void* ws,
                         size_t ws_bytes, hipStream_t stream, bool* handled);
+
+// The kernels each launcher above would enqueue for a call, as text appended to
+// `out` ("name<parameters> grid=... block=..."; several kernels joined by " + ").
+// The describe_* functions that return bool say whether their launcher takes
+// the call; they enqueue nothing.
+const char* dtype_name(int dtype);
+bool describe_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                            int layout, int dtype, const void* values, const void* indices, std::string& out);
+bool describe_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                            int layout, int dtype, std::string& out);
+void describe_stage1_lane_per_bucket(int64_t rows, int64_t k0, int j, int dtype, std::string& out);
+bool describe_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
+                        int layout, int dtype, std::string& out);
+bool describe_multi_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, std::string& out);
+void describe_select(int64_t rows, int64_t k0, int64_t k, int dtype, bool with_workspace, std::string& out);
 
 }  // namespace atk

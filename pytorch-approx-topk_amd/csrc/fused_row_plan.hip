@@ -127,6 +127,18 @@ bool fused_row_takes(const void* x, int64_t rows, int64_t n, int64_t row_stride,
   return plan_for(x, rows, n, row_stride, k0, j, k, layout, dtype).ok;
 }
 
+bool describe_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
+                        int layout, int dtype, std::string& out) {
+  const fused::Plan pl = plan_for(x, rows, n, row_stride, k0, j, k, layout, dtype);
+  if (!pl.ok) return false;
+  out += std::string(pl.in_registers ? "fused_regs_kernel<" : "fused_row_kernel<") + dtype_name(dtype) + ", J=" +
+         std::to_string(j) + ", V=" + std::to_string(pl.vec) + ", pos" + (pl.pos16 ? "16" : "32") +
+         ", PACKED=" + (pl.packed ? "1" : "0") + "> grid=" + std::to_string(rows) + " block=" +
+         std::to_string(64 * pl.waves) + " tiles=" + std::to_string(pl.tiles) + " split=" + std::to_string(pl.split) +
+         " lds=" + std::to_string(pl.lds_bytes) + (pl.in_registers && pl.staged ? " staged" : "");
+  return true;
+}
+
 int launch_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
                      int64_t k, int layout, int dtype, void* values, IndexOut indices, hipStream_t stream,
                      bool* handled) {

@@ -85,6 +85,20 @@ size_t stage1_contig_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j,
   return need;
 }
 
+bool describe_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                            int layout, int dtype, std::string& out) {
+  const int es = elem_bytes(dtype);
+  const int vf = es ? stream::full_vec(es) : 1;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && (row_stride % vf == 0);
+  const contig::Plan pl = contig::make_plan(rows, n, k0, j, layout, dtype, aligned);
+  if (!pl.ok) return false;
+  out += "contig_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + ", V=" +
+         std::to_string(pl.vec) + "> grid=" + std::to_string(rows * (int64_t)pl.geom.groups) + " block=256 chunks=" +
+         std::to_string(pl.geom.chunks) + " slabs=" + std::to_string(pl.geom.slabs);
+  if (pl.geom.slabs > 1) out += " + contig_merge_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + ">";
+  return true;
+}
+
 int launch_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
                          int layout, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
                          hipStream_t stream, bool* handled) {

@@ -87,6 +87,21 @@ static int launch_for_j(const void* x, int64_t rows, int64_t n, int64_t row_stri
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
+const char* dtype_name(int dtype) {
+  switch (dtype) {
+    case ATK_F32: return "f32"; case ATK_F16: return "f16"; case ATK_BF16: return "bf16";
+    case ATK_F64: return "f64"; case ATK_U8: return "u8"; case ATK_I8: return "i8";
+    case ATK_I16: return "i16"; case ATK_I32: return "i32"; case ATK_I64: return "i64";
+  }
+  return "?";
+}
+
+void describe_stage1_lane_per_bucket(int64_t rows, int64_t k0, int j, int dtype, std::string& out) {
+  const int64_t b = j > 0 ? k0 / j : 0;
+  out += "stage1_lane_per_bucket_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) +
+         "> grid=" + std::to_string((b + 255) / 256 * rows) + " block=256";
+}
+
 int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
                                   int64_t row_stride, int64_t k0, int j, int layout,
                                   int dtype, void* values, IndexOut indices,

@@ -140,6 +140,24 @@ size_t stage1_stream_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j,
   return need;
 }
 
+bool describe_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
+                            int layout, int dtype, const void* values, const void* indices, std::string& out) {
+  const int es = elem_bytes(dtype);
+  const int vf = es ? stream::full_vec(es) : 1;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)values % 16 == 0) &&
+                       ((uintptr_t)indices % 16 == 0) && (row_stride % vf == 0);
+  const stream::Plan pl = stream::make_plan(rows, n, k0, j, layout, dtype, aligned);
+  if (!pl.ok) return false;
+  const int loads = pl.packed ? (es == 1 ? 8 : (pl.vec * j <= 8 ? 8 : 4)) : (j <= 2 ? 8 : 4);
+  out += "stream_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) +
+         ", V=" + std::to_string(pl.vec) + ", W=" + std::to_string(pl.waves) + ", U=" + std::to_string(loads) +
+         ", RUN=" + std::to_string(pl.run) + ", PACKED=" + (pl.packed ? "1" : "0") + "> grid=" +
+         std::to_string(rows * (int64_t)pl.slabs * pl.col_tiles) + " block=" + std::to_string(64 * pl.waves) +
+         " fold=" + std::to_string(pl.fold) + " slabs=" + std::to_string(pl.slabs);
+  if (pl.merge) out += " + stream_merge_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + ">";
+  return true;
+}
+
 int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
                          int layout, int dtype, void* values, IndexOut indices, void* ws,
                          size_t ws_bytes, hipStream_t stream, bool* handled) {

@@ -404,6 +404,19 @@ int launch_emit_segments(const void* cand_values, const int64_t* cand_indices, i
   return rc;
 }
 
+bool describe_multi_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, std::string& out) {
+  const MultiPlan pl = plan_multi(rows, k0, k, dtype);
+  if (!pl.use) return false;
+  int index_bits = 1;
+  while (index_bits < 63 && (1ll << index_bits) < index_bound) ++index_bits;
+  const int passes = pl.vc + digit_count(index_bits);
+  const std::string t = dtype_name(dtype);
+  out += "ms_zero_kernel + " + std::to_string(passes) + " x ms_pass_kernel<" + t + "> + ms_count_kernel<" + t +
+         "> + ms_emit_kernel<" + t + "> grid=" + std::to_string(rows * (int64_t)pl.groups) + " block=" +
+         std::to_string(kThreads);
+  return true;
+}
+
 size_t multi_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
   const MultiPlan pl = plan_multi(rows, k0, k, dtype);
   return pl.use ? pl.total : 0;

@@ -173,6 +173,23 @@ size_t select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
   return sp.use ? sp.total : 0;
 }
 
+void describe_select(int64_t rows, int64_t k0, int64_t k, int dtype, bool with_workspace, std::string& out) {
+  const int kb = elem_bytes(dtype) == 8 ? 8 : 4;  // bytes of an order key
+  const bool in_lds = (size_t)k0 * kb <= kMaxKeyLds;
+  int nt = 1024;
+  if (k0 <= 1024) nt = 256;
+  if (rows >= kManyRows) {
+    nt = 64;
+    while (nt < 1024 && (int64_t)nt * 4 < k0) nt *= 2;
+  }
+  const int copies = (in_lds && nt <= 256) ? (nt <= 128 ? 1 : 2) : 8;
+  const SplitPlan sp = plan_split(rows, k0, k);
+  out += "select_kernel<" + std::string(dtype_name(dtype)) + ", KEYS_IN_LDS=" + (in_lds ? "1" : "0") +
+         ", COPIES=" + std::to_string(copies) + "> grid=" + std::to_string(rows) + " block=" + std::to_string(nt);
+  if (sp.use && with_workspace)
+    out += " + ms_emit_kernel<" + std::string(dtype_name(dtype)) + "> grid=" + std::to_string(rows * kSegments);
+}
+
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
                   IndexOut indices, void* ws, size_t ws_bytes, hipStream_t stream) {

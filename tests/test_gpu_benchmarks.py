@@ -1,0 +1,73 @@
+"""The benchmark harness (pytorch-approx-topk_amd/benchmarks/): its timing loop against a direct
+event timing, and its recall figures against the closed form.  Mirrors what the reference's
+benchmarks/measure_speed.py:98-146 and benchmarks/run_recall.py:27-36 compute."""
+import importlib.util
+import os
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _load(name):
+    path = os.path.join(ROOT, "pytorch-approx-topk_amd", "benchmarks", name + ".py")
+    spec = importlib.util.spec_from_file_location("atk_bench_" + name, path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def _direct_us(fn, reps=200):
+    for _ in range(50):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / reps
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_time_calls_agrees_with_a_direct_event_timing(graph):
+    ms = _load("measure_speed")
+    from approx_topk import topk
+    # big enough that the kernel (tens of microseconds) outweighs a launch
+    xs = torch.randn(8, 256, 65536, device="cuda")
+    call = lambda i: topk(xs[i % 8], k=8192, dim=1, j=2)[0]          # noqa: E731
+    mode = dict(graph=True, n_outer=8, n_inner=8) if graph else dict(graph=False, n_outer=64, n_inner=1)
+    durations = ms.time_calls(call, lambda: None, **mode)
+    assert len(durations) == mode["n_outer"] and all(d > 0 for d in durations)
+    got_us = sorted(durations)[len(durations) // 2] * 1e6
+    counter = [0]
+
+    def one():
+        counter[0] += 1
+        return call(counter[0])
+    ref_us = _direct_us(one)           # back-to-back launches: the device time per call once the queue is full
+    assert ref_us / 2.5 < got_us < ref_us * 2.5, (got_us, ref_us)
+    # without the device-side spin an un-graphed single call is timed with the host's enqueue cost inside
+    if not graph:
+        exposed = ms.time_calls(call, lambda: None, hide_launch_cycles=0, **mode)
+        assert sorted(exposed)[len(exposed) // 2] * 1e6 >= got_us * 0.8
+
+
+def test_recalls_against_closed_form():
+    rr = _load("run_recall")
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    xs = torch.rand(rr.N_ROWS, rr.N, device="cuda", generator=gen)
+    for k, j in [(2048, 1), (2048, 2), (4096, 4)]:
+        got = rr.recalls(xs, k, j)
+        expect = rr.closed_form(k, k // j, j)
+        assert abs(got["topk"] - expect) < 0.03, (k, j, got["topk"], expect)
+        assert 0.0 <= got["top50"] <= 1.0 and got["top50"] >= got["topk"] - 1e-6
+        cum = [got["cumulative"][r] for r in sorted(got["cumulative"])]
+        assert all(a >= b for a, b in zip(cum, cum[1:])), cum        # coverage of the first r places cannot grow with r
+        assert cum[0] == 1.0                                          # the maximum is always found
+    # more per bucket at the same k: better recall
+    assert rr.recalls(xs, 2048, 4)["topk"] > rr.recalls(xs, 2048, 1)["topk"]

@@ -78,6 +78,31 @@ def test_native_argument_checks_need_no_gpu():
     assert L.atk_topk_workspace_bytes(3, 100, 16, 1, 8, 0, 0) >= 3 * 16 * 12
 
 
+def test_describe_names_the_planned_kernels():
+    # the planner's choice for a call, as text (no GPU needed: nothing is enqueued)
+    from approx_topk import _native
+    L = _native.lib()
+
+    def describe(rows, n, code, k, j, k_mult, x=4096):
+        buf = ctypes.create_string_buffer(1024)
+        assert L.atk_describe(x, rows, n, n, k * k_mult, j, k, 0, code, 4096, 4096, buf, 1024) == 0
+        return buf.value.decode()
+    c2 = describe(128, 1 << 20, 0, 65536, 2, 1)
+    assert c2.startswith("stream_kernel<f32, J=2, V=4, W=8, U=8, RUN=4, PACKED=0> grid=16384 block=512")
+    c3 = describe(1024, 32768, 1, 2048, 4, 4)
+    assert c3.startswith("fused_regs_kernel<f16, J=4, V=4, pos16, PACKED=1> grid=1024 block=512")
+    c5 = describe(1, 1 << 26, 0, 16384, 4, 2)
+    assert c5.startswith("stream_kernel<f32, J=4") and "stream_merge_kernel" in c5 and "select" in c5
+    # a misaligned input: scalar loads, and two kernels instead of the fused one
+    odd = describe(1024, 32768, 1, 2048, 4, 4, x=4098)
+    assert odd.startswith("stream_kernel<f16, J=4, V=1") and "select_kernel<f16" in odd
+    # truncation and argument checks
+    buf = ctypes.create_string_buffer(8)
+    assert L.atk_describe(4096, 128, 1 << 20, 1 << 20, 65536, 2, 65536, 0, 0, 4096, 4096, buf, 8) == 0
+    assert buf.value == b"stream_"
+    assert L.atk_describe(4096, 1, 8, 8, 6, 4, 6, 0, 0, 4096, 4096, buf, 8) == -2
+
+
 def test_validation_errors_before_device_check():
     from approx_topk import topk
     x = torch.randn(8, 64)
