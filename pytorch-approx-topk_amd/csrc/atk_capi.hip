@@ -277,7 +277,7 @@ int atk_describe(const void* x, int64_t rows, int64_t n, int64_t row_stride, int
       if (k < k0) {
         out += " + ";
         if (!atk::describe_multi_select(rows, k0, k, index_bound_of(n, k0, layout), dtype, out))
-          atk::describe_select(rows, k0, k, dtype, true, out);
+          atk::describe_select(rows, k0, k, index_bound_of(n, k0, layout), dtype, true, out);
       }
     }
   }

@@ -77,6 +77,7 @@ void describe_stage1_lane_per_bucket(int64_t rows, int64_t k0, int j, int dtype,
 bool describe_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
                         int layout, int dtype, std::string& out);
 bool describe_multi_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, std::string& out);
-void describe_select(int64_t rows, int64_t k0, int64_t k, int dtype, bool with_workspace, std::string& out);
+void describe_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, bool with_workspace,
+                     std::string& out);
 
 }  // namespace atk

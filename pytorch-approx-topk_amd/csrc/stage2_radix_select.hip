@@ -8,6 +8,7 @@
 #include "atk_launch.h"
 #include "stage2_select.h"
 
+
 namespace atk {
 
 namespace {
@@ -173,7 +174,9 @@ size_t select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
   return sp.use ? sp.total : 0;
 }
 
-void describe_select(int64_t rows, int64_t k0, int64_t k, int dtype, bool with_workspace, std::string& out) {
+void describe_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, bool with_workspace,
+                     std::string& out) {
+  (void)index_bound;
   const int kb = elem_bytes(dtype) == 8 ? 8 : 4;  // bytes of an order key
   const bool in_lds = (size_t)k0 * kb <= kMaxKeyLds;
   int nt = 1024;

@@ -255,5 +255,103 @@ __device__ __forceinline__ void compact(Sh& sh, uint32_t k0, uint32_t k, Survive
   }
 }
 
+// ---------------------------------------------------------------------------
+// Pieces of a selection over candidates that stay in the registers of the
+// threads that hold them: MSB-first radix passes with 11-bit digits whose
+// histograms (LDS, one atomic add per candidate) one wave reads, and the
+// wave-level scans they need.
+// ---------------------------------------------------------------------------
+namespace regs {
+
+constexpr int kDigitBits = 11;
+constexpr int kBins = 1 << kDigitBits;
+constexpr uint32_t kListMax = 64;
+
+// A histogram holds the count of digit d at word d + (d / 32) * 4, so that the
+// 32 bins every lane of a wave sums (16-byte reads, 144 bytes apart) fall on
+// different LDS banks.
+constexpr uint32_t kHistWords = kBins + kBins / 32 * 4;
+__device__ __forceinline__ uint32_t hist_slot(uint32_t digit) { return digit + ((digit >> 1) & ~15u) / 4u; }
+
+// LDS of a selection over candidates held in registers: two histograms (passes
+// alternate, so that two barriers per pass are enough), then the listed
+// candidates.
+constexpr size_t kListOff = 2 * (size_t)kHistWords * sizeof(uint32_t);
+constexpr size_t kListWords = kListMax + 8;  // rounded up to whole groups of eight when ranking
+constexpr size_t kLdsBytes = kListOff + 2 * kListWords * sizeof(uint64_t);
+
+struct Shared {
+  uint32_t wave_total[kMaxWaves];
+  uint32_t wave_low[kMaxWaves], wave_high[kMaxWaves];  // per-wave smallest and largest key
+  uint32_t list_count;
+  uint32_t digit, need, count;       // what wave 0 found in the last pass
+  uint64_t cut_key, cut_index;       // the cut, when wave 0 ranked a list
+};
+
+// Inclusive prefix sum over the 64 lanes of a wave, in registers.
+__device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
+  // within rows of 16 lanes: shifts by 1, 2, 4, 8 (lanes without a source add 0)
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false);
+  // lane 15 of a row into the next row (rows 1 and 3), then lane 31 into rows 2 and 3
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);
+  return v;
+}
+
+// Smallest and largest of a 32-bit value over the 64 lanes of a wave, in every lane.
+__device__ __forceinline__ uint32_t wave_min(uint32_t v) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t other = (uint32_t)__shfl_xor((int)v, d, kWave);
+    v = other < v ? other : v;
+  }
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_max(uint32_t v) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t other = (uint32_t)__shfl_xor((int)v, d, kWave);
+    v = other > v ? other : v;
+  }
+  return v;
+}
+
+struct Found { uint32_t digit, need, count; };  // wave-uniform
+
+// One wave, all 64 lanes: the bin that holds the need-th entry (1-based) of
+// `total` counted from the best digit down, the rank left within it (again from
+// the best) and its population.
+__device__ __forceinline__ Found find_bin_wave(const uint32_t* hist, uint32_t need_from_top, uint32_t total,
+                                               uint32_t lane) {
+  const uint32_t need = total - need_from_top + 1u;  // counted from the weakest digit up
+  uint32_t mine = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint4 h = *reinterpret_cast<const uint4*>(&hist[lane * 36u + 4u * i]);
+    mine += h.x + h.y + h.z + h.w;
+  }
+  const uint32_t incl = wave_scan(mine);
+  const uint64_t hit = __ballot(incl - mine < need && need <= incl);
+  const int chunk = __builtin_amdgcn_readfirstlane((int)__ffsll((unsigned long long)hit) - 1);
+  const uint32_t before = (uint32_t)__builtin_amdgcn_readlane((int)(incl - mine), chunk);
+  // the 32 bins of that chunk, one per lane
+  const uint32_t bin = lane < 32u ? hist[(uint32_t)chunk * 36u + lane] : 0u;
+  const uint32_t incl2 = wave_scan(bin);
+  const uint32_t left = need - before;
+  const uint64_t hit2 = __ballot(incl2 - bin < left && left <= incl2);
+  const int at = __builtin_amdgcn_readfirstlane((int)__ffsll((unsigned long long)hit2) - 1);
+  Found f;
+  f.digit = (uint32_t)chunk * 32u + (uint32_t)at;
+  f.count = (uint32_t)__builtin_amdgcn_readlane((int)bin, at);
+  // rank within the bin from its weakest member up, turned round
+  f.need = f.count - (left - (uint32_t)__builtin_amdgcn_readlane((int)(incl2 - bin), at)) + 1u;
+  return f;
+}
+
+}  // namespace regs
+
 }  // namespace select
 }  // namespace atk
