@@ -140,7 +140,8 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
     const bool live = has_tile && col < g.b;
     Queue queue;
     if (has_tile) {
-      stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, part == split - 1, queue);
+      if (split > 1) stream::scan_windows<E, J, V, U>(xr, g, col, live, part, split, part == split - 1, queue);
+      else stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, true, queue);
       any_nan |= queue.poisoned();
     }
     if (split > 1) {
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
       __syncthreads();
       if (has_tile && part == 0) {
         for (uint32_t w = 0; w + 1 < split; ++w)
-          queue.fold_in(hand + (size_t)(group * (split - 1) + w) * Queue::kHandBytes, lane);
+          queue.fold_in_interleaved(hand + (size_t)(group * (split - 1) + w) * Queue::kHandBytes, lane);
       }
       if (hand_off == 0) __syncthreads();
     }
@@ -235,7 +236,8 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
   queue.set_position_shift(sizeof(pos_t) == 2 ? (uint32_t)__builtin_clz(g.full_rows | 1u) - 16u : 0u);
   bool any_nan = false;
   if (has_tile) {
-    stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, part == split - 1, queue);
+    if (split > 1) stream::scan_windows<E, J, V, U>(xr, g, col, live, part, split, part == split - 1, queue);
+    else stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, true, queue);
     any_nan = queue.poisoned();
   }
   if (split > 1) {
@@ -244,7 +246,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
     __syncthreads();
     if (has_tile && part == 0) {
       for (uint32_t w = 0; w + 1 < split; ++w)
-        queue.fold_in(hand + (size_t)(tile * (split - 1) + w) * Queue::kHandBytes, lane);
+        queue.fold_in_interleaved(hand + (size_t)(tile * (split - 1) + w) * Queue::kHandBytes, lane);
     }
   }
   // Both histograms start at zero.  Waves that shared a tile must first be done
