@@ -91,10 +91,10 @@ TopkPlan plan_topk(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int la
 // general kernel.
 int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
                int layout, int dtype, void* values, atk::IndexOut indices, void* ws, size_t ws_bytes,
-               hipStream_t stream) {
+               hipStream_t stream, atk::KeyRangeOut* ranges = nullptr) {
   bool handled = false;
   const int rc = atk::launch_stage1_stream(x, rows, n, row_stride, k0, j, layout, dtype, values,
-                                           indices, ws, ws_bytes, stream, &handled);
+                                           indices, ws, ws_bytes, stream, &handled, ranges);
   if (handled || rc != ATK_OK) return rc;
   const int rc2 = atk::launch_stage1_contig(x, rows, n, row_stride, k0, j, layout, dtype, values, indices,
                                             ws, ws_bytes, stream, &handled);
@@ -107,8 +107,11 @@ int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64
 // else one workgroup per row.
 int run_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
                int64_t index_bound, int dtype, void* values, atk::IndexOut indices, void* ws, size_t ws_bytes,
-               hipStream_t stream) {
+               hipStream_t stream, uint32_t range_entries = 0) {
   bool handled = false;
+  const int rcc = atk::launch_chain_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
+                                           indices, ws, ws_bytes, range_entries, stream, &handled);
+  if (handled || rcc != ATK_OK) return rcc;
   const int rc = atk::launch_multi_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
                                           indices, ws, ws_bytes, stream, &handled);
   if (handled || rc != ATK_OK) return rc;
@@ -155,12 +158,15 @@ int do_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t 
   unsigned char* base = static_cast<unsigned char*>(ws);
   void* cand_values = base + p.cand_values_off;
   int64_t* cand_indices = reinterpret_cast<int64_t*>(base + p.cand_indices_off);
+  // a chained select can take the key ranges of the candidates from stage 1's last kernel
+  atk::KeyRangeOut ranges = atk::chain_select_ranges(rows, k0, k, index_bound_of(n, k0, layout), dtype,
+                                                      base + p.select_off, p.select_bytes);
   // the candidates keep int64 indices whatever the output's width
   const int rc1 = run_stage1(x, rows, n, row_stride, k0, j, layout, dtype, cand_values,
-                             atk::IndexOut{cand_indices, 0}, base + p.stage1_off, p.stage1_bytes, stream);
+                             atk::IndexOut{cand_indices, 0}, base + p.stage1_off, p.stage1_bytes, stream, &ranges);
   if (rc1 != ATK_OK) return rc1;
   return run_select(cand_values, cand_indices, rows, k0, k, index_bound_of(n, k0, layout), dtype, values,
-                    indices, base + p.select_off, p.select_bytes, stream);
+                    indices, base + p.select_off, p.select_bytes, stream, ranges.entries);
 }
 
 }  // namespace
@@ -212,7 +218,8 @@ int atk_stage1_i32(const void* x, int64_t rows, int64_t n, int64_t row_stride, i
 size_t atk_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype) {
   const size_t a = atk::multi_select_workspace_bytes(rows, k0, k, dtype);
   const size_t b = atk::select_workspace_bytes(rows, k0, k, dtype);
-  return a > b ? a : b;
+  const size_t c = atk::chain_select_workspace_bytes(rows, k0, k, 0, dtype);
+  return a > b ? (a > c ? a : c) : (b > c ? b : c);
 }
 
 int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0,
@@ -276,7 +283,8 @@ int atk_describe(const void* x, int64_t rows, int64_t n, int64_t row_stride, int
         atk::describe_stage1_lane_per_bucket(rows, k0, j, dtype, out);
       if (k < k0) {
         out += " + ";
-        if (!atk::describe_multi_select(rows, k0, k, index_bound_of(n, k0, layout), dtype, out))
+        if (!atk::describe_chain_select(rows, k0, k, index_bound_of(n, k0, layout), dtype, out) &&
+            !atk::describe_multi_select(rows, k0, k, index_bound_of(n, k0, layout), dtype, out))
           atk::describe_select(rows, k0, k, index_bound_of(n, k0, layout), dtype, true, out);
       }
     }

@@ -18,13 +18,28 @@ int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
                                   int dtype, void* values, IndexOut indices,
                                   hipStream_t stream);
 
+// What stage 1 can leave behind for the chained select of stage2_chain_select.hip,
+// which otherwise spends a launch of its own on it: the smallest and largest
+// order key of shares of every row's candidates, and that select's histogram
+// and row states cleared.  `entries` is set by the stage-1 launcher: shares per
+// row it wrote (0: it wrote nothing and cleared nothing).
+struct KeyRangeOut {
+  uint2* range;             // [rows][entries]
+  uint32_t capacity;        // entries per row that fit
+  uint32_t* hist;           // [rows][hist_words]
+  uint32_t hist_words;
+  uint32_t* state;          // [rows][state_words]
+  uint32_t state_words;
+  uint32_t entries;
+};
+
 // stage1_stream_plan.hip: interleaved layouts with at least j full sub-rows.
 // `*handled` tells whether the shape was accepted; if not, nothing was enqueued.
 size_t stage1_stream_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout,
                                      int dtype);
 int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0,
                          int j, int layout, int dtype, void* values, IndexOut indices, void* ws,
-                         size_t ws_bytes, hipStream_t stream, bool* handled);
+                         size_t ws_bytes, hipStream_t stream, bool* handled, KeyRangeOut* ranges = nullptr);
 
 // stage1_contig_plan.hip: the contiguous layouts, through LDS.  `*handled` as above.
 size_t stage1_contig_workspace_bytes(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype);
@@ -49,6 +64,18 @@ size_t select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int dtype);
 int launch_select(const void* cand_values, const int64_t* cand_indices, int64_t rows,
                   int64_t k0, int64_t k, int64_t index_bound, int dtype, void* values,
                   IndexOut indices, void* ws, size_t ws_bytes, hipStream_t stream);
+
+// stage2_chain_select.hip: few rows of thousands of candidates, several workgroups
+// per row in a chain of three or four launches; needs a workspace.  `*handled` as above.
+size_t chain_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype);
+// Where stage 1 may leave the key ranges for a chained select over workspace `ws`
+// (range == nullptr when that select would not take the call).
+KeyRangeOut chain_select_ranges(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, void* ws,
+                                size_t ws_bytes);
+// `range_entries`: shares per row stage 1 left in the workspace (see KeyRangeOut), or 0.
+int launch_chain_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
+                        int64_t index_bound, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
+                        uint32_t range_entries, hipStream_t stream, bool* handled);
 
 // stage2_multi_select.hip: writes the survivors of every segment of `seg`
 // candidates (`groups` per row) in candidate order, given every row's cut
@@ -77,6 +104,7 @@ void describe_stage1_lane_per_bucket(int64_t rows, int64_t k0, int j, int dtype,
 bool describe_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j, int64_t k,
                         int layout, int dtype, std::string& out);
 bool describe_multi_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, std::string& out);
+bool describe_chain_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, std::string& out);
 void describe_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, bool with_workspace,
                      std::string& out);
 

@@ -45,6 +45,7 @@
 
 #include "atk_device.h"
 #include "atk_launch.h"
+#include "stage2_select.h"
 
 namespace atk {
 namespace stream {
@@ -1114,7 +1115,7 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
     const typename E::raw_t* __restrict__ x, int64_t row_stride,
     const typename E::raw_t* __restrict__ part_values, const uint32_t* __restrict__ part_pos,
     int64_t b, uint32_t slabs, uint32_t cb, uint32_t blocks_per_row,
-    typename E::raw_t* __restrict__ values, const IndexOut indices) {
+    typename E::raw_t* __restrict__ values, const IndexOut indices, const KeyRangeOut ranges) {
   using M = MergeWord<E>;
   using word_t = typename M::word_t;
   constexpr int N = J == 3 ? 4 : J;  // list length of the merge network
@@ -1158,14 +1159,49 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
       merge_best<M, N>(acc, in);
     }
   }
-  if (share != 0 || !live) return;
-  const typename E::raw_t* xr = x + row * row_stride;
-  const int64_t o = (row * b + c) * J;
-  ATK_STATIC_FOR(s, J) {
-    const int64_t index = c + (int64_t)M::pos(acc[N - J + s]) * b;
-    values[o + s] = element_of<E>(acc[N - J + s], xr, index);
-    indices.put(o + s, index);
-  } ATK_STATIC_END;
+  const bool writer = share == 0 && live;
+  if (writer) {
+    const typename E::raw_t* xr = x + row * row_stride;
+    const int64_t o = (row * b + c) * J;
+    ATK_STATIC_FOR(s, J) {
+      const int64_t index = c + (int64_t)M::pos(acc[N - J + s]) * b;
+      values[o + s] = element_of<E>(acc[N - J + s], xr, index);
+      indices.put(o + s, index);
+    } ATK_STATIC_END;
+  }
+  if constexpr (E::key_bits <= 32) {
+    if (ranges.range != nullptr) {
+      // For the chained select that follows (stage2_chain_select.hip): the key
+      // range of this workgroup's results, and this workgroup's share of that
+      // select's histogram and row state cleared.
+      namespace regs = select::regs;
+      __shared__ uint32_t wave_low[kMergeThreads / kWave], wave_high[kMergeThreads / kWave];
+      uint32_t low = ~0u, high = 0;
+      if (writer) {
+        ATK_STATIC_FOR(s, J) {
+          const uint32_t key = (uint32_t)M::key(acc[N - J + s]);
+          low = key < low ? key : low;
+          high = key > high ? key : high;
+        } ATK_STATIC_END;
+      }
+      low = regs::wave_min(low);
+      high = regs::wave_max(high);
+      if (t % kWave == 0) { wave_low[t / kWave] = low; wave_high[t / kWave] = high; }
+      const uint32_t block = blockIdx.x - row32 * blocks_per_row;
+      uint32_t* h = ranges.hist + (size_t)row32 * ranges.hist_words;
+      for (uint32_t i = block * kMergeThreads + t; i < ranges.hist_words; i += blocks_per_row * kMergeThreads) h[i] = 0;
+      if (block == 0 && t < ranges.state_words) ranges.state[(size_t)row32 * ranges.state_words + t] = 0;
+      __syncthreads();
+      if (t == 0) {
+#pragma unroll
+        for (int w = 0; w < kMergeThreads / kWave; ++w) {
+          low = wave_low[w] < low ? wave_low[w] : low;
+          high = wave_high[w] > high ? wave_high[w] : high;
+        }
+        ranges.range[(size_t)row32 * blocks_per_row + block] = make_uint2(low, high);
+      }
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -1190,9 +1226,10 @@ struct Plan {
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype, bool aligned);
 
 // One instance per element type, each in its own translation unit.
+// `ranges`: see KeyRangeOut; may be nullptr.
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j, void* values,
-                 IndexOut indices, void* ws, hipStream_t stream);
+                 IndexOut indices, void* ws, hipStream_t stream, KeyRangeOut* ranges);
 
 }  // namespace stream
 }  // namespace atk

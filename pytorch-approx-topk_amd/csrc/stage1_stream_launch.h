@@ -56,7 +56,7 @@ static int launch_w(const Plan& pl, const typename E::raw_t* x, const Sink<typen
 
 template <typename E, int J>
 static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
-                    const Geom& g, int64_t rows, hipStream_t stream) {
+                    const Geom& g, int64_t rows, hipStream_t stream, KeyRangeOut* ranges) {
   using raw_t = typename E::raw_t;
   constexpr int VF = full_vec((int)sizeof(raw_t));
   const int rc = pl.vec > 1 ? launch_w<E, J, VF>(pl, x, out, g, rows, stream)
@@ -69,16 +69,22 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
   while (cb > 1 && ((int64_t)(cb / 2) >= b || (int64_t)pl.slabs * cb > 32 * kMergeThreads)) cb /= 2;
   const int64_t blocks_per_row = (b + cb - 1) / cb;
   if (blocks_per_row * rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
+  // the merge can leave the key ranges of its results for a chained select
+  KeyRangeOut none{};
+  const bool with_ranges = ranges != nullptr && ranges->range != nullptr && E::key_bits <= 32 &&
+                           blocks_per_row <= (int64_t)ranges->capacity;
+  if (with_ranges) ranges->entries = (uint32_t)blocks_per_row;
   hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)),
                      dim3(kMergeThreads), 0,
                      stream, x, g.row_stride, (const raw_t*)out.part_values, (const uint32_t*)out.part_pos,
-                     b, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices);
+                     b, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices,
+                     with_ranges ? *ranges : none);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
 template <typename E>
 int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride, int j,
-                 void* values, IndexOut indices, void* ws, hipStream_t stream) {
+                 void* values, IndexOut indices, void* ws, hipStream_t stream, KeyRangeOut* ranges) {
   using raw_t = typename E::raw_t;
   Geom g;
   g.row_stride = row_stride; g.b = pl.width;
@@ -92,17 +98,17 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
   out.part_pos = pl.merge ? reinterpret_cast<uint32_t*>(base + pl.part_pos_off) : nullptr;
   const raw_t* xs = static_cast<const raw_t*>(x);
   switch (j) {
-    case 1: return launch_j<E, 1>(pl, xs, out, g, rows, stream);
-    case 2: return launch_j<E, 2>(pl, xs, out, g, rows, stream);
-    case 3: return launch_j<E, 3>(pl, xs, out, g, rows, stream);
-    case 4: return launch_j<E, 4>(pl, xs, out, g, rows, stream);
+    case 1: return launch_j<E, 1>(pl, xs, out, g, rows, stream, ranges);
+    case 2: return launch_j<E, 2>(pl, xs, out, g, rows, stream, ranges);
+    case 3: return launch_j<E, 3>(pl, xs, out, g, rows, stream, ranges);
+    case 4: return launch_j<E, 4>(pl, xs, out, g, rows, stream, ranges);
   }
   return ATK_ERR_J;
 }
 
 #define ATK_INSTANTIATE_STREAM(DT)                                                          \
   template int launch_typed<Elem<DT>>(const Plan&, const void*, int64_t, int64_t, int, void*, \
-                                      IndexOut, void*, hipStream_t);
+                                      IndexOut, void*, hipStream_t, KeyRangeOut*);
 
 }  // namespace stream
 }  // namespace atk

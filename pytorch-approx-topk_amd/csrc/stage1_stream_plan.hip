@@ -160,7 +160,7 @@ bool describe_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_
 
 int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t k0, int j,
                          int layout, int dtype, void* values, IndexOut indices, void* ws,
-                         size_t ws_bytes, hipStream_t stream, bool* handled) {
+                         size_t ws_bytes, hipStream_t stream, bool* handled, KeyRangeOut* ranges) {
   const int es = elem_bytes(dtype);
   const int vf = es ? stream::full_vec(es) : 1;
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)values % 16 == 0) &&
@@ -172,7 +172,7 @@ int launch_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_str
   int rc = ATK_ERR_DTYPE;
   ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
                    rc = stream::launch_typed<E>(pl, x, rows, row_stride, j, values, indices, ws,
-                                                stream));
+                                                stream, ranges));
   return rc;
 }
 

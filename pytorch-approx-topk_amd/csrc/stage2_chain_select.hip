@@ -1,0 +1,487 @@
+// Stage 2 for few rows of many candidates (thousands to tens of thousands per
+// row): the exact top-k selection spread over several workgroups per row in a
+// short chain of launches.
+//
+// One workgroup per row (stage2_radix_select.hip) pushes all of a row's
+// candidates through one CU: about 0.8 us per thousand candidates, 25 us at
+// 32768.  Here a row is cut into segments of kSegment candidates, one workgroup
+// each, and up to four small kernels follow one another on the stream:
+//
+//   range:   every workgroup finds the smallest and largest order key of its
+//            segment (and clears its share of the row's histogram).
+//   hist:    from the row's key range every workgroup works out the first bit
+//            in which any two keys differ, takes the 11 bits from there down as
+//            the digit, and adds its segment's digit histogram to the row's.
+//            (The candidates of a top-k lie close together: the leading key
+//            bits, sign and exponent, are the same in all of them.)
+//   refine:  every workgroup finds the digit B of the k-th best from the row's
+//            histogram, counts its candidates above B and lists those in B
+//            (order key, inverted index and candidate number) in the row's list.
+//   emit:    every workgroup ranks the listed candidates (a few dozen, as a rule)
+//            to find the weakest survivor, offsets by the survivors of the
+//            segments before it and writes its own in candidate order.
+//
+// A candidate is the 64-bit word (order key, inverted index): a greater word is a
+// better candidate and no two are equal, so that ties go to the lower index.
+// A row whose digit B holds more candidates than the list takes is selected by
+// its first workgroup alone, with the block-wide radix select over all of its
+// candidates.  When stage 1 ends in a kernel that can leave the key ranges of
+// its results behind (KeyRangeOut), the range launch is skipped.  Results are
+// those of the one-workgroup kernel: same survivors, same order.
+#include "atk_device.h"
+#include "atk_launch.h"
+#include "stage2_select.h"
+
+namespace atk {
+namespace {
+
+namespace regs = select::regs;
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / select::kWave;
+constexpr int kPerThread = 4;
+constexpr uint32_t kSegment = kThreads * kPerThread;  // candidates per workgroup
+constexpr uint32_t kListCap = 2048;                   // listed candidates a row can hold
+constexpr uint32_t kRankDirect = 256;                 // lists up to this size are ranked by counting
+
+// Per-row words in the workspace.
+struct RowState {
+  uint32_t list_count;  // candidates appended to the list (may exceed kListCap: then the row is left to the fallback)
+  uint32_t digit;       // B
+  uint32_t need;        // members of B that belong to the result
+  uint32_t count;       // members of B
+  uint32_t shift, bits; // the digit is (key >> shift) & ((1 << bits) - 1)
+  uint32_t fallback;    // != 0: the one-workgroup kernel takes this row
+  uint32_t unused;
+};
+
+// Shares per row whose key ranges the workspace has room for: the chain's own
+// segments, or the workgroups of a stage-1 kernel that left them (KeyRangeOut).
+constexpr uint32_t kRangeCapacity = 4096;
+
+struct ChainPlan {
+  bool use;
+  uint32_t groups;  // workgroups per row
+  uint32_t range_capacity;
+  size_t range_off, hist_off, state_off, above_off, list_word_off, list_at_off, total;
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Thread t of a workgroup holds candidates first + u * kThreads, u = 0..kPerThread-1, of its row.
+template <typename E>
+__device__ __forceinline__ void load_keys(const typename E::raw_t* __restrict__ cv, uint32_t first, uint32_t k0,
+                                          uint32_t (&key)[kPerThread], bool (&valid)[kPerThread]) {
+  typename E::raw_t raw[kPerThread];
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    valid[u] = first + u * kThreads < k0;
+    raw[u] = valid[u] ? cv[first + u * kThreads] : (typename E::raw_t)0;
+  }
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) key[u] = (uint32_t)E::key(raw[u]);
+}
+
+template <typename E>
+__global__ __launch_bounds__(kThreads) void chain_range_kernel(const typename E::raw_t* __restrict__ cand_values,
+                                                               uint32_t k0, uint32_t groups, uint2* __restrict__ range,
+                                                               uint32_t* __restrict__ hist, RowState* __restrict__ state) {
+  __shared__ uint32_t wave_low[kWaves], wave_high[kWaves];
+  const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
+  const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
+  uint32_t key[kPerThread];
+  bool valid[kPerThread];
+  load_keys<E>(cand_values + (int64_t)row * k0, g * kSegment + tid, k0, key, valid);
+  uint32_t low = ~0u, high = 0;
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    if (valid[u]) {
+      low = key[u] < low ? key[u] : low;
+      high = key[u] > high ? key[u] : high;
+    }
+  }
+  low = regs::wave_min(low);
+  high = regs::wave_max(high);
+  if (lane == 0) { wave_low[wave] = low; wave_high[wave] = high; }
+  // this workgroup's share of the row's histogram, and the row's state
+  uint32_t* h = hist + (size_t)row * regs::kHistWords;
+  for (uint32_t i = g * kThreads + tid; i < regs::kHistWords; i += groups * kThreads) h[i] = 0;
+  if (g == 0 && tid == 0) state[row] = RowState{0, 0, 0, 0, 0, 0, 0, 0};
+  __syncthreads();
+  if (tid == 0) {
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      low = wave_low[w] < low ? wave_low[w] : low;
+      high = wave_high[w] > high ? wave_high[w] : high;
+    }
+    range[(size_t)row * groups + g] = make_uint2(low, high);
+  }
+}
+
+// The digit position of a row from the key ranges of its segments.  Whole
+// workgroup; `red` is 2 * kWaves words of LDS; ends with a barrier.
+__device__ __forceinline__ void digit_of_row(const uint2* __restrict__ range, uint32_t groups, uint32_t* red,
+                                             uint32_t& shift, uint32_t& bits) {
+  const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
+  uint32_t low = ~0u, high = 0;
+  for (uint32_t g = tid; g < groups; g += kThreads) {
+    const uint2 r = range[g];
+    low = r.x < low ? r.x : low;
+    high = r.y > high ? r.y : high;
+  }
+  low = regs::wave_min(low);
+  high = regs::wave_max(high);
+  if (lane == 0) { red[wave] = low; red[kWaves + wave] = high; }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    low = red[w] < low ? red[w] : low;
+    high = red[kWaves + w] > high ? red[kWaves + w] : high;
+  }
+  const uint32_t differing = low >= high ? 0u : 32u - (uint32_t)__builtin_clz(low ^ high);
+  bits = differing < (uint32_t)regs::kDigitBits ? differing : (uint32_t)regs::kDigitBits;
+  shift = differing - bits;
+}
+
+template <typename E>
+__global__ __launch_bounds__(kThreads) void chain_hist_kernel(const typename E::raw_t* __restrict__ cand_values,
+                                                              uint32_t k0, uint32_t groups,
+                                                              const uint2* __restrict__ range, uint32_t entries,
+                                                              uint32_t* __restrict__ hist) {
+  __shared__ uint32_t local[regs::kHistWords];
+  __shared__ uint32_t red[2 * kWaves];
+  const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
+  const uint32_t tid = threadIdx.x;
+  uint32_t key[kPerThread];
+  bool valid[kPerThread];
+  load_keys<E>(cand_values + (int64_t)row * k0, g * kSegment + tid, k0, key, valid);
+  for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = 0;
+  uint32_t shift, bits;
+  digit_of_row(range + (size_t)row * entries, entries, red, shift, bits);  // (its barrier also covers the clearing)
+  const uint32_t dmask = (1u << bits) - 1u;
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u)
+    if (valid[u]) atomicAdd(&local[regs::hist_slot((key[u] >> shift) & dmask)], 1u);
+  __syncthreads();
+  uint32_t* h = hist + (size_t)row * regs::kHistWords;
+  for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) {
+    const uint32_t c = local[i];
+    if (c != 0) atomicAdd(&h[i], c);
+  }
+}
+
+template <typename E>
+__global__ __launch_bounds__(kThreads) void chain_refine_kernel(
+    const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
+    uint32_t k, uint32_t groups, const uint2* __restrict__ range, uint32_t entries,
+    const uint32_t* __restrict__ hist, RowState* __restrict__ state, uint32_t* __restrict__ above,
+    uint64_t* __restrict__ list_word, uint32_t* __restrict__ list_at) {
+  __shared__ __align__(16) uint32_t local[regs::kHistWords];
+  __shared__ regs::Found found;
+  __shared__ uint32_t wave_above[kWaves];
+  __shared__ uint32_t red[2 * kWaves];
+  const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
+  const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
+  const uint32_t first = g * kSegment + tid;
+  // everything this workgroup reads is asked for at once: keys, indices, the row's histogram and ranges
+  uint32_t key[kPerThread], inv[kPerThread];
+  bool valid[kPerThread];
+  load_keys<E>(cand_values + (int64_t)row * k0, first, k0, key, valid);
+  const int64_t* ci = cand_indices + (int64_t)row * k0;
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) inv[u] = valid[u] ? ~(uint32_t)ci[first + u * kThreads] : 0u;
+  const uint32_t* h = hist + (size_t)row * regs::kHistWords;
+  for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = h[i];
+  uint32_t shift, bits;
+  digit_of_row(range + (size_t)row * entries, entries, red, shift, bits);  // (its barrier also publishes `local`)
+  const uint32_t dmask = (1u << bits) - 1u;
+  if (wave == 0) {
+    const regs::Found f = regs::find_bin_wave(local, k, k0, lane);
+    if (lane == 0) found = f;
+  }
+  __syncthreads();
+  const regs::Found f = found;
+  uint32_t mine = 0;
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    if (!valid[u]) continue;
+    const uint32_t d = (key[u] >> shift) & dmask;
+    // survivors known now: above B, and all of B when none of it is cut
+    mine += (d > f.digit || (d == f.digit && f.need == f.count)) ? 1u : 0u;
+    if (d == f.digit && f.need != f.count) {  // the digit is cut: its members are ranked later
+      const uint32_t slot = atomicAdd(&state[row].list_count, 1u);
+      if (slot < kListCap) {
+        list_word[(size_t)row * kListCap + slot] = ((uint64_t)key[u] << 32) | (uint64_t)inv[u];
+        list_at[(size_t)row * kListCap + slot] = first + u * kThreads;
+      }
+    }
+  }
+  const uint32_t incl = regs::wave_scan(mine);
+  if (lane == select::kWave - 1) wave_above[wave] = incl;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t total = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) total += wave_above[w];
+    above[(size_t)row * groups + g] = total;
+    if (g == 0) {
+      RowState* s = &state[row];
+      s->digit = f.digit; s->need = f.need; s->count = f.count; s->shift = shift; s->bits = bits;
+      s->fallback = (f.need != f.count && f.count > kListCap) ? 1u : 0u;
+    }
+  }
+}
+
+template <typename E>
+__global__ __launch_bounds__(kThreads) void chain_emit_kernel(
+    const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
+    uint32_t k, uint32_t groups, int index_bits, const RowState* __restrict__ state,
+    const uint32_t* __restrict__ above, const uint64_t* __restrict__ list_word,
+    const uint32_t* __restrict__ list_at, typename E::raw_t* __restrict__ values, const IndexOut indices) {
+  using raw_t = typename E::raw_t;
+  using key_t = typename E::key_t;
+  extern __shared__ __align__(16) unsigned char dyn_lds[];
+  __shared__ select::SharedT<2> sh;
+  __shared__ uint64_t cut_word;
+  __shared__ uint32_t listed_before;
+  __shared__ uint32_t wave_kept[kPerThread][kWaves];
+  const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
+  const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
+  // asked for before the row's state is known: the start of the list (most lists end within it) and
+  // the survivors counted for the segments before this one
+  const uint64_t early_word = list_word[(size_t)row * kListCap + tid];
+  const uint32_t early_at = list_at[(size_t)row * kListCap + tid];
+  uint32_t counted = 0;
+  for (uint32_t p = tid; p < g; p += kThreads) counted += above[(size_t)row * groups + p];
+  const RowState s = state[row];
+  if (s.fallback != 0) {
+    // The cut digit holds more candidates than the list: the row's first
+    // workgroup runs the block-wide radix select of stage2_select.h over all of
+    // the row's candidates, read from global memory (slow, but only rows with
+    // thousands of equal keys around the cut come here).
+    if (g != 0) return;
+    const raw_t* rv = cand_values + (int64_t)row * k0;
+    const int64_t* ri = cand_indices + (int64_t)row * k0;
+    auto key_at = [&](uint32_t i) -> key_t { return E::key(rv[i]); };
+    auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)ri[i]; };
+    const select::Cut<key_t> whole = select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
+    auto survives = [&](uint32_t i) -> bool {
+      const key_t key = key_at(i);
+      if (key != whole.T) return key > whole.T;
+      return whole.index_cut == ~0ull || index_at(i) <= whole.index_cut;
+    };
+    struct Candidate { raw_t value; int64_t index; };
+    raw_t* out_values = values + (int64_t)row * k;
+    const int64_t out_first = (int64_t)row * k;
+    select::compact(
+        sh, k0, k, survives, [&](uint32_t i) { return Candidate{rv[i], ri[i]}; },
+        [&](uint32_t, uint32_t o, const Candidate& c) { out_values[o] = c.value; indices.put(out_first + o, c.index); });
+    return;
+  }
+  const bool cut_digit = s.need != s.count;  // else every member of B survives
+  const uint32_t n = cut_digit ? s.count : 0u;
+  uint64_t* words = reinterpret_cast<uint64_t*>(dyn_lds);
+  uint32_t* ats = reinterpret_cast<uint32_t*>(dyn_lds + (size_t)kListCap * sizeof(uint64_t));
+  const uint32_t first = g * kSegment + tid;
+  const raw_t* cv = cand_values + (int64_t)row * k0;
+  const int64_t* ci = cand_indices + (int64_t)row * k0;
+  // this thread's candidates: elements, keys and indices
+  raw_t raw[kPerThread];
+  uint32_t inv[kPerThread];
+  bool valid[kPerThread];
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    valid[u] = first + u * kThreads < k0;
+    raw[u] = valid[u] ? cv[first + u * kThreads] : (raw_t)0;
+    inv[u] = valid[u] ? ~(uint32_t)ci[first + u * kThreads] : 0u;
+  }
+  // entries past the list's end count as beating nothing (ranking reads the list in groups of eight)
+  words[tid] = tid < n ? early_word : 0ull;
+  ats[tid] = tid < n ? early_at : ~0u;
+  for (uint32_t i = tid + kThreads; i < ((n + 7u) & ~7u); i += kThreads) {
+    words[i] = i < n ? list_word[(size_t)row * kListCap + i] : 0ull;
+    ats[i] = i < n ? list_at[(size_t)row * kListCap + i] : ~0u;
+  }
+  if (tid == 0) { cut_word = 0; listed_before = 0; }
+  __syncthreads();
+  uint64_t cut = 0;  // the weakest surviving member of B (0: all of them survive)
+  if (n != 0) {
+    if (n <= kRankDirect) {
+      // thread t counts the entries better than entry t: the need-th best is the cut
+      if (tid < n) {
+        const uint64_t mine = words[tid];
+        uint32_t better = 0;
+        for (uint32_t m = 0; m < n; m += 8) {
+          uint64_t got[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) got[e] = words[m + e];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) better += got[e] > mine ? 1u : 0u;
+        }
+        if (better + 1 == s.need) cut_word = mine;
+      }
+      __syncthreads();
+      cut = cut_word;
+    } else {
+      // a longer list: the block-wide radix select over its words (all distinct)
+      auto key_at = [&](uint32_t i) -> uint64_t { return words[i]; };
+      auto index_at = [&](uint32_t) -> uint64_t { return 0; };
+      cut = select::find_cut<uint64_t, 64>(sh, n, s.need, 1, key_at, index_at).T;
+    }
+    // listed survivors of the segments before this one
+    uint32_t before = 0;
+    for (uint32_t i = tid; i < n; i += kThreads) before += (ats[i] < g * kSegment && words[i] >= cut) ? 1u : 0u;
+    before = regs::wave_scan(before);
+    if (lane == select::kWave - 1 && before != 0) atomicAdd(&listed_before, before);
+  }
+  // survivors of this thread, counted per u and wave (candidate order: u, then thread)
+  const uint32_t dmask = (1u << s.bits) - 1u;
+  bool sel[kPerThread];
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    const uint32_t key = (uint32_t)E::key(raw[u]);
+    const uint32_t d = (key >> s.shift) & dmask;
+    sel[u] = valid[u] && (d > s.digit || (d == s.digit && (((uint64_t)key << 32) | inv[u]) >= cut));
+    const uint64_t m = __ballot(sel[u]);
+    if (lane == 0) wave_kept[u][wave] = (uint32_t)__popcll(m);
+  }
+  // survivors of the segments before this one that the refine step counted
+  counted = regs::wave_scan(counted);
+  if (lane == select::kWave - 1 && counted != 0) atomicAdd(&listed_before, counted);
+  __syncthreads();
+  uint32_t base = listed_before;
+  raw_t* ov = values + (int64_t)row * k;
+  const int64_t oi = (int64_t)row * k;
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    uint32_t o = base;
+    for (int w = 0; w < kWaves; ++w) {
+      if ((uint32_t)w < wave) o += wave_kept[u][w];
+    }
+    const uint64_t m = __ballot(sel[u]);
+    if (sel[u]) {
+      const uint32_t at = o + select::rank_in(m);
+      if (at < k) {
+        ov[at] = raw[u];
+        indices.put(oi + at, (int64_t)(uint32_t)~inv[u]);
+      }
+    }
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) base += wave_kept[u][w];
+  }
+}
+
+// Rows for which the chain beats one workgroup per row: few rows (one workgroup
+// per row already fills the GPU with many), enough candidates that a single CU
+// is what bounds them, keys of at most 32 bits and indices below 2^31.
+constexpr int64_t kChainMinCandidates = 8192;
+constexpr int64_t kChainMaxCandidates = 1 << 17;
+constexpr int64_t kChainMaxRows = 64;
+
+ChainPlan plan_chain(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype) {
+  ChainPlan pl{};
+  pl.use = false;
+  const int es = elem_bytes(dtype);
+  if (es == 0 || es > 4 || rows <= 0 || rows > kChainMaxRows || k <= 0 || k >= k0) return pl;
+  if (k0 < kChainMinCandidates || k0 > kChainMaxCandidates || index_bound > 0x7fffffffll) return pl;
+  pl.groups = (uint32_t)((k0 + kSegment - 1) / kSegment);
+  pl.range_off = 0;
+  pl.range_capacity = pl.groups > kRangeCapacity ? pl.groups : kRangeCapacity;
+  pl.hist_off = align_up((size_t)rows * pl.range_capacity * sizeof(uint2), 256);
+  pl.state_off = pl.hist_off + align_up((size_t)rows * regs::kHistWords * sizeof(uint32_t), 256);
+  pl.above_off = pl.state_off + align_up((size_t)rows * sizeof(RowState), 256);
+  pl.list_word_off = pl.above_off + align_up((size_t)rows * pl.groups * sizeof(uint32_t), 256);
+  pl.list_at_off = pl.list_word_off + align_up((size_t)rows * kListCap * sizeof(uint64_t), 256);
+  pl.total = pl.list_at_off + align_up((size_t)rows * kListCap * sizeof(uint32_t), 256);
+  pl.use = true;
+  return pl;
+}
+
+template <typename E>
+int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64_t* cand_indices, int64_t rows,
+                       int64_t k0, int64_t k, int index_bits, void* values, IndexOut indices, void* ws,
+                       uint32_t range_entries, hipStream_t stream) {
+  using raw_t = typename E::raw_t;
+  if constexpr (sizeof(typename E::key_t) == 4) {
+    unsigned char* base = static_cast<unsigned char*>(ws);
+    uint2* range = reinterpret_cast<uint2*>(base + pl.range_off);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(base + pl.hist_off);
+    RowState* state = reinterpret_cast<RowState*>(base + pl.state_off);
+    uint32_t* above = reinterpret_cast<uint32_t*>(base + pl.above_off);
+    uint64_t* list_word = reinterpret_cast<uint64_t*>(base + pl.list_word_off);
+    uint32_t* list_at = reinterpret_cast<uint32_t*>(base + pl.list_at_off);
+    const raw_t* cv = static_cast<const raw_t*>(cand_values);
+    const dim3 grid((unsigned)(rows * pl.groups)), block(kThreads);
+    const size_t emit_lds = (size_t)kListCap * (sizeof(uint64_t) + sizeof(uint32_t));
+    uint32_t entries = range_entries;
+    if (entries == 0) {  // stage 1 left no key ranges
+      hipLaunchKernelGGL((chain_range_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups, range, hist,
+                         state);
+      entries = pl.groups;
+    }
+    hipLaunchKernelGGL((chain_hist_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups,
+                       (const uint2*)range, entries, hist);
+    hipLaunchKernelGGL((chain_refine_kernel<E>), grid, block, 0, stream, cv, cand_indices, (uint32_t)k0, (uint32_t)k,
+                       pl.groups, (const uint2*)range, entries, (const uint32_t*)hist, state, above, list_word,
+                       list_at);
+    hipLaunchKernelGGL((chain_emit_kernel<E>), grid, block, emit_lds, stream, cv, cand_indices, (uint32_t)k0,
+                       (uint32_t)k, pl.groups, index_bits, (const RowState*)state, (const uint32_t*)above,
+                       (const uint64_t*)list_word, (const uint32_t*)list_at, static_cast<raw_t*>(values), indices);
+    return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+  } else {
+    (void)pl; (void)cand_values; (void)cand_indices; (void)rows; (void)k0; (void)k; (void)index_bits; (void)values;
+    (void)indices; (void)ws; (void)range_entries; (void)stream;
+    return ATK_ERR_DTYPE;
+  }
+}
+
+}  // namespace
+
+size_t chain_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype) {
+  const ChainPlan pl = plan_chain(rows, k0, k, index_bound, dtype);
+  return pl.use ? pl.total : 0;
+}
+
+bool describe_chain_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, std::string& out) {
+  const ChainPlan pl = plan_chain(rows, k0, k, index_bound, dtype);
+  if (!pl.use) return false;
+  const std::string t = dtype_name(dtype);
+  out += "[chain_range_kernel<" + t + "> unless stage 1 left the key ranges] + chain_hist_kernel<" + t +
+         "> + chain_refine_kernel<" + t +
+         "> + chain_emit_kernel<" + t + "> grid=" + std::to_string(rows * (int64_t)pl.groups) + " block=" +
+         std::to_string(kThreads);
+  return true;
+}
+
+KeyRangeOut chain_select_ranges(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, void* ws,
+                                size_t ws_bytes) {
+  KeyRangeOut out{};
+  const ChainPlan pl = plan_chain(rows, k0, k, index_bound, dtype);
+  if (!pl.use || !ws || ws_bytes < pl.total || (uintptr_t)ws % 16 != 0) return out;
+  unsigned char* base = static_cast<unsigned char*>(ws);
+  out.range = reinterpret_cast<uint2*>(base + pl.range_off);
+  out.capacity = pl.range_capacity;
+  out.hist = reinterpret_cast<uint32_t*>(base + pl.hist_off);
+  out.hist_words = regs::kHistWords;
+  out.state = reinterpret_cast<uint32_t*>(base + pl.state_off);
+  out.state_words = (uint32_t)(sizeof(RowState) / sizeof(uint32_t));
+  return out;
+}
+
+int launch_chain_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
+                        int64_t index_bound, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
+                        uint32_t range_entries, hipStream_t stream, bool* handled) {
+  const ChainPlan pl = plan_chain(rows, k0, k, index_bound, dtype);
+  *handled = pl.use;
+  if (!pl.use) return ATK_OK;
+  if (!ws || ws_bytes < pl.total || (uintptr_t)ws % 16 != 0) return ATK_ERR_WORKSPACE;
+  int index_bits = 1;
+  while (index_bits < 63 && (1ll << index_bits) < index_bound) ++index_bits;
+  int rc = ATK_ERR_DTYPE;
+  ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
+                   rc = launch_chain_typed<E>(pl, cand_values, cand_indices, rows, k0, k, index_bits, values, indices,
+                                              ws, range_entries, stream));
+  return rc;
+}
+
+}  // namespace atk

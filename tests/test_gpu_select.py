@@ -91,3 +91,61 @@ def test_topk_with_many_candidates(dtype, interleaved):
     v, i = topk(x.cuda(), 32768, -1, j=2, k_mult=4, interleaved=interleaved)   # 131072 candidates per row
     ev, ei = oracle.topk(x, 32768, -1, j=2, k_mult=4, interleaved=interleaved)
     assert_same(v, i, ev, ei, f"{dtype} interleaved={interleaved}")
+
+
+# ---- few rows of thousands of candidates: several workgroups per row in a short chain of launches ----
+
+def _chain_case(rows_spec, k0, k, dtype, bound=1 << 21, seed=0):
+    """rows_spec: per row 'spread' (distinct values), 'ties' (seven values), 'equal' (one value),
+    'steps' (blocks of equal values: the cut digit is shared by thousands)."""
+    g = torch.Generator().manual_seed(seed)
+    rows = []
+    for kind in rows_spec:
+        if kind == "spread":
+            r = torch.randn(k0, generator=g) if dtype.is_floating_point else torch.randint(-30000, 30000, (k0,), generator=g)
+        elif kind == "ties":
+            r = torch.randint(-3, 4, (k0,), generator=g)
+        elif kind == "equal":
+            r = torch.full((k0,), 2.0)
+        else:
+            r = (torch.arange(k0) // 3000).float()[torch.randperm(k0, generator=g)]
+        rows.append(r.to(dtype))
+    cv = torch.stack(rows)
+    ci = torch.stack([torch.randperm(bound, generator=g)[:k0] for _ in rows_spec])
+    v, i = _select(cv, ci, k, bound)
+    ev, ei = oracle.stage2(cv, ci, k)
+    assert_same(v, i, ev, ei, f"{rows_spec} k0={k0} k={k} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.int32, torch.int16, torch.uint8])
+@pytest.mark.parametrize("k0,k", [(8192, 2048), (32768, 16384), (20000, 1), (9001, 9000), (131072, 5000)])
+def test_chain_select_rows_of_every_kind_together(dtype, k0, k):
+    # rows that end by prefix, by a ranked list, by a long list and by the whole-row fallback, in one call
+    kinds = ["spread", "ties", "equal", "steps", "spread"]
+    if dtype == torch.uint8:
+        kinds = ["ties", "equal", "steps"]
+    _chain_case(kinds, k0, k, dtype, seed=k0 + k)
+
+
+def test_chain_select_needs_no_cut_when_the_digit_belongs_whole():
+    # k falls exactly on a boundary between two values: every member of the cut digit survives
+    k0 = 16384
+    cv = torch.cat([torch.full((6000,), 3.0), torch.full((k0 - 6000,), 1.0)])[torch.randperm(k0)].reshape(1, k0)
+    ci = torch.randperm(1 << 20)[:k0].reshape(1, k0)
+    v, i = _select(cv, ci, 6000, 1 << 20)
+    ev, ei = oracle.stage2(cv, ci, 6000)
+    assert_same(v, i, ev, ei, "whole digit")
+
+
+def test_chain_select_after_stage1_takes_the_key_ranges_from_the_merge():
+    # one long row through the operator: slabs + merge (which leaves the key ranges) + chained select
+    from approx_topk import topk
+    g = torch.Generator().manual_seed(7)
+    x = torch.randint(-2000, 2000, (2, 1 << 22), generator=g).float() / 16        # many ties
+    v, i = topk(x.cuda(), 8192, -1, j=4, k_mult=2)
+    ev, ei = oracle.topk(x, 8192, -1, j=4, k_mult=2)
+    assert_same(v, i, ev, ei, "two long rows")
+    x16 = x.half()
+    v, i = topk(x16.cuda(), 4096, -1, j=2, k_mult=4)
+    ev, ei = oracle.topk(x16, 4096, -1, j=2, k_mult=4)
+    assert_same(v, i, ev, ei, "two long fp16 rows")
