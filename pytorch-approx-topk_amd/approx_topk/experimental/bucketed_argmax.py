@@ -43,23 +43,29 @@ def topk_torch(xs: Tensor, k: int, dim: int, interleaved: bool) -> tuple[Tensor,
 
 
 def _batch_contiguous(x: Tensor) -> Tensor:
-    """``x`` itself when its rows are unit-stride and uniformly spaced in memory
-    (so the whole batch is addressed by one row stride), else a contiguous copy.
+    """``x`` itself when one row pitch addresses the whole batch, else a copy.
 
-    E.g. for shape (2, 3, 4): strides (12, 4, 1) and (15, 5, 1) pass unchanged;
-    (*, *, 2), (13, 4, 1) and (4, 8, 1) are copied.
+    The native entry takes a base pointer, a row count and one pitch in
+    elements, so every row must start ``pitch`` elements after the previous one
+    in flattened batch order, with ``pitch >= n`` and unit stride inside a row.
+    A [6, 5, 8] tensor sliced to ``[:, :, :7]`` qualifies (pitch 8); sliced to
+    ``[:, :4]`` it does not (the rows of consecutive outer entries are 16 apart,
+    not 8), nor does any view whose last stride is not 1.
     """
-    strides, shape = x.stride(), x.shape
-    if strides[-1] != 1:
+    if x.stride(-1) != 1:
         return x.contiguous()
-    if x.ndim >= 2:
-        step = strides[-2]
-        if step < shape[-1]:
+    if x.ndim == 1:
+        return x
+    pitch = x.stride(-2)
+    if pitch < x.shape[-1]:
+        return x.contiguous()
+    # Row (i0, .., i_{m-1}) must sit at pitch * flat(i): dimension d's stride is
+    # then the pitch times the number of rows under one step of d.
+    rows_under = 1
+    for size, stride in zip(reversed(x.shape[:-1]), reversed(x.stride()[:-1])):
+        if size > 1 and stride != pitch * rows_under:
             return x.contiguous()
-        for d in range(x.ndim - 2, -1, -1):
-            if strides[d] != step:
-                return x.contiguous()
-            step *= shape[d]
+        rows_under *= size
     return x
 
 
