@@ -107,10 +107,10 @@ int run_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64
 // else one workgroup per row.
 int run_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
                int64_t index_bound, int dtype, void* values, atk::IndexOut indices, void* ws, size_t ws_bytes,
-               hipStream_t stream, uint32_t range_entries = 0) {
+               hipStream_t stream, uint32_t range_entries = 0, bool hist_done = false) {
   bool handled = false;
   const int rcc = atk::launch_chain_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
-                                           indices, ws, ws_bytes, range_entries, stream, &handled);
+                                           indices, ws, ws_bytes, range_entries, hist_done, stream, &handled);
   if (handled || rcc != ATK_OK) return rcc;
   const int rc = atk::launch_multi_select(cand_values, cand_indices, rows, k0, k, index_bound, dtype, values,
                                           indices, ws, ws_bytes, stream, &handled);
@@ -166,7 +166,7 @@ int do_topk(const void* x, int64_t rows, int64_t n, int64_t row_stride, int64_t 
                              atk::IndexOut{cand_indices, 0}, base + p.stage1_off, p.stage1_bytes, stream, &ranges);
   if (rc1 != ATK_OK) return rc1;
   return run_select(cand_values, cand_indices, rows, k0, k, index_bound_of(n, k0, layout), dtype, values,
-                    indices, base + p.select_off, p.select_bytes, stream, ranges.entries);
+                    indices, base + p.select_off, p.select_bytes, stream, ranges.entries, ranges.hist_done != 0);
 }
 
 }  // namespace

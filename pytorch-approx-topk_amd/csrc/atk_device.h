@@ -114,7 +114,7 @@ struct IndexOut {
   }
 };
 
-__host__ __device__ inline int elem_bytes(int dtype) {
+__host__ __device__ constexpr int elem_bytes(int dtype) {
   switch (dtype) {
     case ATK_F32: case ATK_I32: return 4;
     case ATK_F16: case ATK_BF16: case ATK_I16: return 2;
@@ -123,6 +123,10 @@ __host__ __device__ inline int elem_bytes(int dtype) {
   }
   return 0;
 }
+
+// The element type code of a traits type.
+template <typename E> struct DtypeOf;
+template <int DT> struct DtypeOf<Elem<DT>> { static constexpr int value = DT; };
 
 // ---------------------------------------------------------------------------
 // Bucket geometry: first position, stride between members and member count of

@@ -19,10 +19,13 @@ int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
                                   hipStream_t stream);
 
 // What stage 1 can leave behind for the chained select of stage2_chain_select.hip,
-// which otherwise spends a launch of its own on it: the smallest and largest
-// order key of shares of every row's candidates, and that select's histogram
-// and row states cleared.  `entries` is set by the stage-1 launcher: shares per
-// row it wrote (0: it wrote nothing and cleared nothing).
+// which otherwise spends launches of its own on it: the smallest and largest
+// order key of shares of every row's candidates (shares of a superset of them
+// will do: the ranges only say which key bits all candidates have in common),
+// that select's row states cleared, and its histogram either cleared or
+// already filled with the candidates' digits.  The stage-1 launcher sets
+// `entries`: shares per row it wrote (0: it wrote nothing and cleared nothing),
+// and `hist_done`: the histogram holds the candidates' digits.
 struct KeyRangeOut {
   uint2* range;             // [rows][entries]
   uint32_t capacity;        // entries per row that fit
@@ -31,6 +34,7 @@ struct KeyRangeOut {
   uint32_t* state;          // [rows][state_words]
   uint32_t state_words;
   uint32_t entries;
+  uint32_t hist_done;
 };
 
 // stage1_stream_plan.hip: interleaved layouts with at least j full sub-rows.
@@ -72,10 +76,11 @@ size_t chain_select_workspace_bytes(int64_t rows, int64_t k0, int64_t k, int64_t
 // (range == nullptr when that select would not take the call).
 KeyRangeOut chain_select_ranges(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype, void* ws,
                                 size_t ws_bytes);
-// `range_entries`: shares per row stage 1 left in the workspace (see KeyRangeOut), or 0.
+// `range_entries`: shares per row stage 1 left in the workspace (see KeyRangeOut), or 0;
+// `hist_done`: it also filled the histogram.
 int launch_chain_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
                         int64_t index_bound, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
-                        uint32_t range_entries, hipStream_t stream, bool* handled);
+                        uint32_t range_entries, bool hist_done, hipStream_t stream, bool* handled);
 
 // stage2_multi_select.hip: writes the survivors of every segment of `seg`
 // candidates (`groups` per row) in candidate order, given every row's cut

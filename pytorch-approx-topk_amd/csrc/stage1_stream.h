@@ -554,9 +554,140 @@ template <typename E, int J, int V> struct ByteQueue {
   template <int VI, int SI> __device__ __forceinline__ uint32_t position() const { return 0xffffffu - (q[VI][SI] & 0xffffffu); }
 };
 
+// Wide form for fp32 with two or more entries per column: an entry is one
+// 64-bit word read as a double, the element's bits in the high half and the
+// sub-row number below it, so that a push is J v_max_f64 and J-1 v_min_f64
+// (both issue at the rate of 32-bit operations on this part) where the general
+// form takes J compares and about 4 J selects.
+//
+// Why the order is right: a non-NaN float's bits, taken as the high word of a
+// double (sign, then 8 + 3 bits as exponent, then mantissa), order as the float
+// does, and the exponent field is all ones only for some NaNs, so that every
+// word is a finite double.  Among equal elements the lower sub-row must win:
+// the low word holds ~sub-row under a positive element and sub-row under a
+// negative one (where a larger magnitude is the smaller double).  -0.0 is read
+// as +0.0 first (x + 0.0f), as the order has them equal; entries with a zero
+// element are re-read from the row at the end to learn their sign
+// (`fix_zeros`).  Loads are screened for NaN as in the general form.  The empty
+// entry is the double -inf, below every word.
+__device__ __forceinline__ double max_f64(double a, double b) {
+  double r;
+  asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ double min_f64(double a, double b) {
+  double r;
+  asm("v_min_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+template <typename E, int J, int V> struct WideQueue {
+  using raw_t = typename E::raw_t;
+  static_assert(std::is_same<E, Elem<ATK_F32>>::value && J >= 2, "wide queues hold fp32 elements");
+  static constexpr size_t kHandBytes = (size_t)V * J * kWave * 8;
+
+  double q[V][J];
+  uint64_t nan_mask;   // lanes that loaded a NaN; wave-uniform
+  uint32_t neg_zeros;  // bit v*J+s: entry (v, s) is a -0.0 (set by fix_zeros)
+
+  __device__ static __forceinline__ double empty() { return __longlong_as_double((long long)0xfff0000000000000ull); }
+  __device__ static __forceinline__ uint32_t high(double w) { return (uint32_t)((uint64_t)__double_as_longlong(w) >> 32); }
+  __device__ static __forceinline__ uint32_t low(double w) { return (uint32_t)(uint64_t)__double_as_longlong(w); }
+  // `c`: the element with -0.0 already read as +0.0; np: ~sub-row
+  __device__ static __forceinline__ double word(float c, uint32_t np) {
+    const uint32_t hi = __float_as_uint(c);
+    const uint32_t lo = np ^ (uint32_t)((int32_t)hi >> 31);
+    return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+  }
+  __device__ static __forceinline__ void insert(double (&col)[J], double w) {
+    ATK_STATIC_FOR(s, J - 1) { col[s] = max_f64(col[s], min_f64(w, col[s + 1])); } ATK_STATIC_END;
+    col[J - 1] = max_f64(col[J - 1], w);
+  }
+
+  __device__ __forceinline__ void reset() {
+    ATK_STATIC_FOR(e, V * J) { q[e / J][e % J] = empty(); } ATK_STATIC_END;
+    nan_mask = 0;
+    neg_zeros = 0;
+  }
+  __device__ __forceinline__ void set_position_shift(uint32_t) {}
+  __device__ __forceinline__ int sel_constant_bits() const { return 0; }
+
+  template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
+    const uint32_t np = ~p;
+    float c[V];
+    ATK_STATIC_FOR(v, V) { c[v] = __uint_as_float(pk.e[v]) + 0.0f; } ATK_STATIC_END;
+    ATK_STATIC_FOR(h, V / 2) { nan_mask |= __ballot(__builtin_isunordered(c[2 * h], c[2 * h + 1])); } ATK_STATIC_END;
+    if constexpr (V % 2 != 0) nan_mask |= __ballot(__builtin_isunordered(c[V - 1], c[V - 1]));
+    ATK_STATIC_FOR(v, V) { insert(q[v], word(c[v], np)); } ATK_STATIC_END;
+  }
+  template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
+    const float c = __uint_as_float(raw) + 0.0f;
+    nan_mask |= __ballot(valid && __builtin_isunordered(c, c));
+    insert(q[VI], valid ? word(c, ~p) : empty());
+  }
+  __device__ __forceinline__ bool poisoned() const { return nan_mask != 0; }
+
+  __device__ __forceinline__ void hand_over(unsigned char* area, uint32_t lane) const {
+    double* h = reinterpret_cast<double*>(area);
+    ATK_STATIC_FOR(e, V * J) { h[e * kWave + lane] = q[e / J][e % J]; } ATK_STATIC_END;
+  }
+  // (entry words carry their whole order: any arrival order gives the same queue)
+  __device__ __forceinline__ void fold_in(const unsigned char* area, uint32_t lane) {
+    const double* h = reinterpret_cast<const double*>(area);
+    ATK_STATIC_FOR(e, V * J) { insert(q[e / J], h[e * kWave + lane]); } ATK_STATIC_END;
+  }
+  __device__ __forceinline__ void fold_in_interleaved(const unsigned char* area, uint32_t lane) { fold_in(area, lane); }
+  // Final entries with a zero element are re-read from the row to learn their
+  // sign.  `col` is the lane's first column; call once, after the last fold, by live lanes.
+  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__ xr, int64_t b, int64_t col) {
+    bool any = false;
+    ATK_STATIC_FOR(e, V * J) { any |= high(q[e / J][e % J]) == 0u; } ATK_STATIC_END;
+    if (__ballot(any) == 0) return;
+    ATK_STATIC_FOR(e, V * J) {
+      if (high(q[e / J][e % J]) == 0u) {
+        const uint32_t p = ~low(q[e / J][e % J]);
+        if (xr[(int64_t)p * b + col + e / J] == 0x80000000u) neg_zeros |= 1u << e;
+      }
+    } ATK_STATIC_END;
+  }
+  template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return E::key(high(q[VI][SI])); }
+  using sel_t = typename E::key_t;
+  static constexpr int sel_bits = E::key_bits;
+  template <int VI, int SI> __device__ __forceinline__ sel_t sel_key() const { return key<VI, SI>(); }
+  template <int VI, int SI> __device__ __forceinline__ uint2 staged(uint32_t column) const {
+    return make_uint2(high(q[VI][SI]), (position<VI, SI>() << 16) | column);
+  }
+  struct Unstaged { raw_t raw; uint32_t sub_row, column; bool reread; };
+  __device__ __forceinline__ Unstaged unstage(uint2 w) const {
+    return Unstaged{w.x, w.y >> 16, w.y & 0xffffu, w.x == 0u};
+  }
+  template <int VI, int SI> __device__ __forceinline__ raw_t raw() const {
+    return (neg_zeros >> (VI * J + SI)) & 1u ? 0x80000000u : high(q[VI][SI]);
+  }
+  template <int VI, int SI> __device__ __forceinline__ uint32_t position() const {
+    const uint32_t hi = high(q[VI][SI]);
+    return ~(low(q[VI][SI]) ^ (uint32_t)((int32_t)hi >> 31));
+  }
+};
+
+// fewest entries per column from which fp32 queues take the wide form
+constexpr int kWideFromJ = 2;
+
+// Loads a lane keeps in flight (the kernels' U).  Packed queues: bytes load 8
+// per lane and keep few registers per entry.  General queues of J >= 3 leave
+// registers for four; the wide fp32 queues cost half the instructions, so
+// that their scan waits on memory and eight pay (fp32 [1, 2^26], 8192 buckets,
+// J = 4: 50.6 -> 48.2 us; sixteen: 66.8 us).
+__host__ __device__ constexpr int loads_in_flight(int dtype, int j, int vec, bool packed) {
+  if (packed) return elem_bytes(dtype) == 1 ? 8 : (vec * j <= 8 ? 8 : 4);
+  return (j <= 2 || (dtype == ATK_F32 && j >= kWideFromJ)) ? 8 : 4;
+}
+
 template <typename E, int J, int V, bool PACKED, bool SHIFTED = false>
 using QueueFor = std::conditional_t<
-    !PACKED, CmpQueue<E, J, V>,
+    !PACKED,
+    std::conditional_t<std::is_same<E, Elem<ATK_F32>>::value && (J >= kWideFromJ), WideQueue<E, (J >= 2 ? J : 2), V>,
+                       CmpQueue<E, J, V>>,
     std::conditional_t<sizeof(typename E::raw_t) == 1, ByteQueue<E, J, V>, PackedQueue<E, J, V, SHIFTED>>>;
 
 // Shape of one launch; passed to the kernels by value.  With few buckets the
@@ -1038,7 +1169,8 @@ __device__ __forceinline__ void fold_columns_exact(const typename E::raw_t* __re
 // PACKED: packed 16-bit queues.
 template <typename E, int J, int V, int W, int U, int RUN, bool PACKED>
 __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) void stream_kernel(
-    const typename E::raw_t* __restrict__ x, const Sink<typename E::raw_t> out, const Geom g) {
+    const typename E::raw_t* __restrict__ x, const Sink<typename E::raw_t> out, const Geom g,
+    const KeyRangeOut ranges) {
   using raw_t = typename E::raw_t;
   using Queue = QueueFor<E, J, V, PACKED>;
   constexpr int kTileCols = kWave * V;
@@ -1083,6 +1215,9 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
       for (int w = 0; w < W - 1; ++w) queue.fold_in(lds + (size_t)w * Queue::kHandBytes, lane);
     }
   }
+  // order keys of what this workgroup leaves, smallest and largest (all keys
+  // when that is not worked out: any range that holds them will do)
+  uint32_t low = 0u, high = ~0u;
   if (g.fold > 1) {
     if (redo) {
       fold_columns_exact<E, J>(xr, g, out, row, slab, s0, s1, last_slab, lane);
@@ -1090,15 +1225,40 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
       if (live) queue.fix_zeros(xr, g.b, col);
       fold_columns<E, J, V>(xr, g, out, row, slab, col, live, lane, queue, lds);
     }
-    return;
-  }
-  if (!live) return;
-  if (redo) {
+  } else if (!live) {
+    low = ~0u; high = 0u;
+  } else if (redo) {
     exact_columns<E, J, V>(xr, g, out, row, slab, col, s0, W > 1 ? s1 : p1, last_slab);
-    return;
+  } else {
+    queue.fix_zeros(xr, g.b, col);
+    emit<E, J, V>(g, out, row, slab, col, queue);
+    if constexpr (E::key_bits <= 32) {
+      if (ranges.range != nullptr) {
+        low = ~0u; high = 0u;
+        ATK_STATIC_FOR(e, V * J) {
+          const uint32_t key = (uint32_t)queue.template key<e / J, e % J>();
+          low = key < low ? key : low;
+          high = key > high ? key : high;
+        } ATK_STATIC_END;
+      }
+    }
   }
-  queue.fix_zeros(xr, g.b, col);
-  emit<E, J, V>(g, out, row, slab, col, queue);
+  if constexpr (E::key_bits <= 32) {
+    if (ranges.range != nullptr) {
+      // For the chained select that follows the merge of the slabs
+      // (stage2_chain_select.hip): the key range of this workgroup's queues, and
+      // this workgroup's share of that select's histogram and row state cleared.
+      namespace regs = select::regs;
+      low = regs::wave_min(low);
+      high = regs::wave_max(high);
+      const uint32_t blocks_per_row = g.slabs * g.col_tiles;
+      const uint32_t block = slab * g.col_tiles + col_tile;
+      if (lane == 0) ranges.range[(size_t)row * blocks_per_row + block] = make_uint2(low, high);
+      uint32_t* h = ranges.hist + (size_t)row * ranges.hist_words;
+      for (uint32_t i = block * kWave + lane; i < ranges.hist_words; i += blocks_per_row * kWave) h[i] = 0;
+      if (block == 0 && lane < ranges.state_words) ranges.state[(size_t)row * ranges.state_words + lane] = 0;
+    }
+  }
 }
 
 // Folds the slabs' partial queues of every bucket into the final result under
@@ -1171,34 +1331,29 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
   }
   if constexpr (E::key_bits <= 32) {
     if (ranges.range != nullptr) {
-      // For the chained select that follows (stage2_chain_select.hip): the key
-      // range of this workgroup's results, and this workgroup's share of that
-      // select's histogram and row state cleared.
+      // For the chained select that follows (stage2_chain_select.hip): the
+      // digits of this workgroup's results added to the row's histogram, which
+      // the scanning kernel cleared; the digit's place comes from the key ranges
+      // that kernel left of its queues, which hold every result.
+      // (Added up in LDS first: thousands of atomic adds to the few words of
+      // the crowded digits, straight to memory, take hundreds of microseconds.)
       namespace regs = select::regs;
-      __shared__ uint32_t wave_low[kMergeThreads / kWave], wave_high[kMergeThreads / kWave];
-      uint32_t low = ~0u, high = 0;
-      if (writer) {
+      __shared__ uint32_t red[2 * kMergeThreads / kWave];
+      __shared__ uint32_t local[regs::kHistWords];
+      for (uint32_t i = t; i < (uint32_t)regs::kHistWords; i += kMergeThreads) local[i] = 0;
+      uint32_t low, shift;
+      regs::digit_of_row<kMergeThreads>(ranges.range + (size_t)row32 * ranges.entries, ranges.entries, red, low, shift);
+      if (writer) {  // (the barrier in digit_of_row also covers the clearing)
         ATK_STATIC_FOR(s, J) {
           const uint32_t key = (uint32_t)M::key(acc[N - J + s]);
-          low = key < low ? key : low;
-          high = key > high ? key : high;
+          atomicAdd(&local[regs::hist_slot((key - low) >> shift)], 1u);
         } ATK_STATIC_END;
       }
-      low = regs::wave_min(low);
-      high = regs::wave_max(high);
-      if (t % kWave == 0) { wave_low[t / kWave] = low; wave_high[t / kWave] = high; }
-      const uint32_t block = blockIdx.x - row32 * blocks_per_row;
-      uint32_t* h = ranges.hist + (size_t)row32 * ranges.hist_words;
-      for (uint32_t i = block * kMergeThreads + t; i < ranges.hist_words; i += blocks_per_row * kMergeThreads) h[i] = 0;
-      if (block == 0 && t < ranges.state_words) ranges.state[(size_t)row32 * ranges.state_words + t] = 0;
       __syncthreads();
-      if (t == 0) {
-#pragma unroll
-        for (int w = 0; w < kMergeThreads / kWave; ++w) {
-          low = wave_low[w] < low ? wave_low[w] : low;
-          high = wave_high[w] > high ? wave_high[w] : high;
-        }
-        ranges.range[(size_t)row32 * blocks_per_row + block] = make_uint2(low, high);
+      uint32_t* h = ranges.hist + (size_t)row32 * ranges.hist_words;
+      for (uint32_t i = t; i < (uint32_t)regs::kHistWords; i += kMergeThreads) {
+        const uint32_t c = local[i];
+        if (c != 0) atomicAdd(&h[i], c);
       }
     }
   }

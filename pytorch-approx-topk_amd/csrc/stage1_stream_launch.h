@@ -9,47 +9,46 @@ namespace stream {
 
 template <typename E, int J, int V, int W, int RUN>
 static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
-                      const Geom& g, dim3 grid, hipStream_t stream) {
-  constexpr int U = J <= 2 ? 8 : 4;
+                      const Geom& g, dim3 grid, hipStream_t stream, const KeyRangeOut& left) {
+  constexpr int U = loads_in_flight(DtypeOf<E>::value, J, V, false);
   if constexpr (PackedKey<E>::available) {
     if (pl.packed) {
-      // loads in flight: bytes load 8 per lane and keep few registers per entry
-      constexpr int UP = sizeof(typename E::raw_t) == 1 ? 8 : (V * J <= 8 ? 8 : 4);
-      hipLaunchKernelGGL((stream_kernel<E, J, V, W, UP, RUN, true>), grid, dim3(kWave * W), 0, stream, x, out, g);
+      constexpr int UP = loads_in_flight(DtypeOf<E>::value, J, V, true);
+      hipLaunchKernelGGL((stream_kernel<E, J, V, W, UP, RUN, true>), grid, dim3(kWave * W), 0, stream, x, out, g, left);
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }
   }
-  hipLaunchKernelGGL((stream_kernel<E, J, V, W, U, RUN, false>), grid, dim3(kWave * W), 0, stream, x, out, g);
+  hipLaunchKernelGGL((stream_kernel<E, J, V, W, U, RUN, false>), grid, dim3(kWave * W), 0, stream, x, out, g, left);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 
 template <typename E, int J, int V, int W>
 static int launch_one(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
-                      const Geom& g, int64_t rows, hipStream_t stream) {
+                      const Geom& g, int64_t rows, hipStream_t stream, const KeyRangeOut& left) {
   const int64_t groups = rows * (int64_t)pl.slabs * pl.col_tiles;
   if (groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   const dim3 grid((unsigned)groups);
   // combinations the planner never picks are not compiled
   if constexpr (merge_lds_bytes(V, J, W, sizeof(typename Cmp<E>::cmp_t)) <= kMergeLdsLimit) {
     if constexpr (V > 1) {  // exact short runs exist for the vector kernels only
-      if (pl.run == 4) return launch_run<E, J, V, W, 4>(pl, x, out, g, grid, stream);
-      if (pl.run == 8) return launch_run<E, J, V, W, 8>(pl, x, out, g, grid, stream);
+      if (pl.run == 4) return launch_run<E, J, V, W, 4>(pl, x, out, g, grid, stream, left);
+      if (pl.run == 8) return launch_run<E, J, V, W, 8>(pl, x, out, g, grid, stream, left);
     }
-    return launch_run<E, J, V, W, 0>(pl, x, out, g, grid, stream);
+    return launch_run<E, J, V, W, 0>(pl, x, out, g, grid, stream, left);
   } else {
-    (void)x; (void)out; (void)g; (void)stream;
+    (void)x; (void)out; (void)g; (void)stream; (void)left;
     return ATK_ERR_ARG;
   }
 }
 
 template <typename E, int J, int V>
 static int launch_w(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
-                    const Geom& g, int64_t rows, hipStream_t stream) {
+                    const Geom& g, int64_t rows, hipStream_t stream, const KeyRangeOut& left) {
   switch (pl.waves) {
-    case 1: return launch_one<E, J, V, 1>(pl, x, out, g, rows, stream);
-    case 2: return launch_one<E, J, V, 2>(pl, x, out, g, rows, stream);
-    case 4: return launch_one<E, J, V, 4>(pl, x, out, g, rows, stream);
-    case 8: return launch_one<E, J, V, 8>(pl, x, out, g, rows, stream);
+    case 1: return launch_one<E, J, V, 1>(pl, x, out, g, rows, stream, left);
+    case 2: return launch_one<E, J, V, 2>(pl, x, out, g, rows, stream, left);
+    case 4: return launch_one<E, J, V, 4>(pl, x, out, g, rows, stream, left);
+    case 8: return launch_one<E, J, V, 8>(pl, x, out, g, rows, stream, left);
   }
   return ATK_ERR_ARG;
 }
@@ -59,8 +58,18 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
                     const Geom& g, int64_t rows, hipStream_t stream, KeyRangeOut* ranges) {
   using raw_t = typename E::raw_t;
   constexpr int VF = full_vec((int)sizeof(raw_t));
-  const int rc = pl.vec > 1 ? launch_w<E, J, VF>(pl, x, out, g, rows, stream)
-                            : launch_w<E, J, 1>(pl, x, out, g, rows, stream);
+  // Kernels that end in the merge of slabs can leave a chained select its key
+  // ranges (one per scanning workgroup) and its histogram.
+  KeyRangeOut left{};
+  const int64_t scan_blocks = (int64_t)pl.slabs * pl.col_tiles;  // per row
+  if (ranges != nullptr && ranges->range != nullptr && E::key_bits <= 32 && pl.merge &&
+      scan_blocks <= (int64_t)ranges->capacity) {
+    ranges->entries = (uint32_t)scan_blocks;
+    ranges->hist_done = 1;
+    left = *ranges;
+  }
+  const int rc = pl.vec > 1 ? launch_w<E, J, VF>(pl, x, out, g, rows, stream, left)
+                            : launch_w<E, J, 1>(pl, x, out, g, rows, stream, left);
   if (rc != ATK_OK || !pl.merge) return rc;
   const int64_t b = pl.width / pl.fold;  // buckets
   // buckets per workgroup: a power of two, no more than there are, and few
@@ -69,16 +78,10 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
   while (cb > 1 && ((int64_t)(cb / 2) >= b || (int64_t)pl.slabs * cb > 32 * kMergeThreads)) cb /= 2;
   const int64_t blocks_per_row = (b + cb - 1) / cb;
   if (blocks_per_row * rows > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
-  // the merge can leave the key ranges of its results for a chained select
-  KeyRangeOut none{};
-  const bool with_ranges = ranges != nullptr && ranges->range != nullptr && E::key_bits <= 32 &&
-                           blocks_per_row <= (int64_t)ranges->capacity;
-  if (with_ranges) ranges->entries = (uint32_t)blocks_per_row;
   hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)),
                      dim3(kMergeThreads), 0,
                      stream, x, g.row_stride, (const raw_t*)out.part_values, (const uint32_t*)out.part_pos,
-                     b, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices,
-                     with_ranges ? *ranges : none);
+                     b, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices, left);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 

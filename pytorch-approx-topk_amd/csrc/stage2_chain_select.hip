@@ -9,11 +9,11 @@
 //
 //   range:   every workgroup finds the smallest and largest order key of its
 //            segment (and clears its share of the row's histogram).
-//   hist:    from the row's key range every workgroup works out the first bit
-//            in which any two keys differ, takes the 11 bits from there down as
-//            the digit, and adds its segment's digit histogram to the row's.
-//            (The candidates of a top-k lie close together: the leading key
-//            bits, sign and exponent, are the same in all of them.)
+//   hist:    from the row's key range every workgroup works out the digit of
+//            a key, the leading 11 bits of its offset from the row's smallest
+//            key within the span of the row's keys, and adds its segment's
+//            digit histogram to the row's.  (The candidates of a top-k lie
+//            close together: their keys span a small part of the key space.)
 //   refine:  every workgroup finds the digit B of the k-th best from the row's
 //            histogram, counts its candidates above B and lists those in B
 //            (order key, inverted index and candidate number) in the row's list.
@@ -25,9 +25,10 @@
 // better candidate and no two are equal, so that ties go to the lower index.
 // A row whose digit B holds more candidates than the list takes is selected by
 // its first workgroup alone, with the block-wide radix select over all of its
-// candidates.  When stage 1 ends in a kernel that can leave the key ranges of
-// its results behind (KeyRangeOut), the range launch is skipped.  Results are
-// those of the one-workgroup kernel: same survivors, same order.
+// candidates.  When stage 1 ends in kernels that can leave key ranges and the
+// histogram behind (KeyRangeOut: the streaming kernel's slabs and their merge),
+// the range and hist launches are skipped.  Results are those of the
+// one-workgroup kernel: same survivors, same order.
 #include "atk_device.h"
 #include "atk_launch.h"
 #include "stage2_select.h"
@@ -50,7 +51,7 @@ struct RowState {
   uint32_t digit;       // B
   uint32_t need;        // members of B that belong to the result
   uint32_t count;       // members of B
-  uint32_t shift, bits; // the digit is (key >> shift) & ((1 << bits) - 1)
+  uint32_t shift, low;  // the digit is (key - low) >> shift
   uint32_t fallback;    // != 0: the one-workgroup kernel takes this row
   uint32_t unused;
 };
@@ -118,31 +119,6 @@ __global__ __launch_bounds__(kThreads) void chain_range_kernel(const typename E:
   }
 }
 
-// The digit position of a row from the key ranges of its segments.  Whole
-// workgroup; `red` is 2 * kWaves words of LDS; ends with a barrier.
-__device__ __forceinline__ void digit_of_row(const uint2* __restrict__ range, uint32_t groups, uint32_t* red,
-                                             uint32_t& shift, uint32_t& bits) {
-  const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
-  uint32_t low = ~0u, high = 0;
-  for (uint32_t g = tid; g < groups; g += kThreads) {
-    const uint2 r = range[g];
-    low = r.x < low ? r.x : low;
-    high = r.y > high ? r.y : high;
-  }
-  low = regs::wave_min(low);
-  high = regs::wave_max(high);
-  if (lane == 0) { red[wave] = low; red[kWaves + wave] = high; }
-  __syncthreads();
-#pragma unroll
-  for (int w = 0; w < kWaves; ++w) {
-    low = red[w] < low ? red[w] : low;
-    high = red[kWaves + w] > high ? red[kWaves + w] : high;
-  }
-  const uint32_t differing = low >= high ? 0u : 32u - (uint32_t)__builtin_clz(low ^ high);
-  bits = differing < (uint32_t)regs::kDigitBits ? differing : (uint32_t)regs::kDigitBits;
-  shift = differing - bits;
-}
-
 template <typename E>
 __global__ __launch_bounds__(kThreads) void chain_hist_kernel(const typename E::raw_t* __restrict__ cand_values,
                                                               uint32_t k0, uint32_t groups,
@@ -156,12 +132,11 @@ __global__ __launch_bounds__(kThreads) void chain_hist_kernel(const typename E::
   bool valid[kPerThread];
   load_keys<E>(cand_values + (int64_t)row * k0, g * kSegment + tid, k0, key, valid);
   for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = 0;
-  uint32_t shift, bits;
-  digit_of_row(range + (size_t)row * entries, entries, red, shift, bits);  // (its barrier also covers the clearing)
-  const uint32_t dmask = (1u << bits) - 1u;
+  uint32_t low, shift;
+  regs::digit_of_row<kThreads>(range + (size_t)row * entries, entries, red, low, shift);  // (its barrier also covers the clearing)
 #pragma unroll
   for (int u = 0; u < kPerThread; ++u)
-    if (valid[u]) atomicAdd(&local[regs::hist_slot((key[u] >> shift) & dmask)], 1u);
+    if (valid[u]) atomicAdd(&local[regs::hist_slot((key[u] - low) >> shift)], 1u);
   __syncthreads();
   uint32_t* h = hist + (size_t)row * regs::kHistWords;
   for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) {
@@ -192,9 +167,8 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
   for (int u = 0; u < kPerThread; ++u) inv[u] = valid[u] ? ~(uint32_t)ci[first + u * kThreads] : 0u;
   const uint32_t* h = hist + (size_t)row * regs::kHistWords;
   for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = h[i];
-  uint32_t shift, bits;
-  digit_of_row(range + (size_t)row * entries, entries, red, shift, bits);  // (its barrier also publishes `local`)
-  const uint32_t dmask = (1u << bits) - 1u;
+  uint32_t low, shift;
+  regs::digit_of_row<kThreads>(range + (size_t)row * entries, entries, red, low, shift);  // (its barrier also publishes `local`)
   if (wave == 0) {
     const regs::Found f = regs::find_bin_wave(local, k, k0, lane);
     if (lane == 0) found = f;
@@ -205,7 +179,7 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
 #pragma unroll
   for (int u = 0; u < kPerThread; ++u) {
     if (!valid[u]) continue;
-    const uint32_t d = (key[u] >> shift) & dmask;
+    const uint32_t d = (key[u] - low) >> shift;
     // survivors known now: above B, and all of B when none of it is cut
     mine += (d > f.digit || (d == f.digit && f.need == f.count)) ? 1u : 0u;
     if (d == f.digit && f.need != f.count) {  // the digit is cut: its members are ranked later
@@ -226,7 +200,7 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
     above[(size_t)row * groups + g] = total;
     if (g == 0) {
       RowState* s = &state[row];
-      s->digit = f.digit; s->need = f.need; s->count = f.count; s->shift = shift; s->bits = bits;
+      s->digit = f.digit; s->need = f.need; s->count = f.count; s->shift = shift; s->low = low;
       s->fallback = (f.need != f.count && f.count > kListCap) ? 1u : 0u;
     }
   }
@@ -335,12 +309,11 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
     if (lane == select::kWave - 1 && before != 0) atomicAdd(&listed_before, before);
   }
   // survivors of this thread, counted per u and wave (candidate order: u, then thread)
-  const uint32_t dmask = (1u << s.bits) - 1u;
   bool sel[kPerThread];
 #pragma unroll
   for (int u = 0; u < kPerThread; ++u) {
     const uint32_t key = (uint32_t)E::key(raw[u]);
-    const uint32_t d = (key >> s.shift) & dmask;
+    const uint32_t d = (key - s.low) >> s.shift;
     sel[u] = valid[u] && (d > s.digit || (d == s.digit && (((uint64_t)key << 32) | inv[u]) >= cut));
     const uint64_t m = __ballot(sel[u]);
     if (lane == 0) wave_kept[u][wave] = (uint32_t)__popcll(m);
@@ -400,7 +373,7 @@ ChainPlan plan_chain(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, i
 template <typename E>
 int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64_t* cand_indices, int64_t rows,
                        int64_t k0, int64_t k, int index_bits, void* values, IndexOut indices, void* ws,
-                       uint32_t range_entries, hipStream_t stream) {
+                       uint32_t range_entries, bool hist_done, hipStream_t stream) {
   using raw_t = typename E::raw_t;
   if constexpr (sizeof(typename E::key_t) == 4) {
     unsigned char* base = static_cast<unsigned char*>(ws);
@@ -419,8 +392,9 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
                          state);
       entries = pl.groups;
     }
-    hipLaunchKernelGGL((chain_hist_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups,
-                       (const uint2*)range, entries, hist);
+    if (!hist_done || range_entries == 0)
+      hipLaunchKernelGGL((chain_hist_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups,
+                         (const uint2*)range, entries, hist);
     hipLaunchKernelGGL((chain_refine_kernel<E>), grid, block, 0, stream, cv, cand_indices, (uint32_t)k0, (uint32_t)k,
                        pl.groups, (const uint2*)range, entries, (const uint32_t*)hist, state, above, list_word,
                        list_at);
@@ -430,7 +404,7 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
     return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
   } else {
     (void)pl; (void)cand_values; (void)cand_indices; (void)rows; (void)k0; (void)k; (void)index_bits; (void)values;
-    (void)indices; (void)ws; (void)range_entries; (void)stream;
+    (void)indices; (void)ws; (void)range_entries; (void)hist_done; (void)stream;
     return ATK_ERR_DTYPE;
   }
 }
@@ -446,8 +420,8 @@ bool describe_chain_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bo
   const ChainPlan pl = plan_chain(rows, k0, k, index_bound, dtype);
   if (!pl.use) return false;
   const std::string t = dtype_name(dtype);
-  out += "[chain_range_kernel<" + t + "> unless stage 1 left the key ranges] + chain_hist_kernel<" + t +
-         "> + chain_refine_kernel<" + t +
+  out += "[chain_range_kernel<" + t + "> + chain_hist_kernel<" + t +
+         "> unless stage 1 left key ranges and histogram] + chain_refine_kernel<" + t +
          "> + chain_emit_kernel<" + t + "> grid=" + std::to_string(rows * (int64_t)pl.groups) + " block=" +
          std::to_string(kThreads);
   return true;
@@ -470,7 +444,7 @@ KeyRangeOut chain_select_ranges(int64_t rows, int64_t k0, int64_t k, int64_t ind
 
 int launch_chain_select(const void* cand_values, const int64_t* cand_indices, int64_t rows, int64_t k0, int64_t k,
                         int64_t index_bound, int dtype, void* values, IndexOut indices, void* ws, size_t ws_bytes,
-                        uint32_t range_entries, hipStream_t stream, bool* handled) {
+                        uint32_t range_entries, bool hist_done, hipStream_t stream, bool* handled) {
   const ChainPlan pl = plan_chain(rows, k0, k, index_bound, dtype);
   *handled = pl.use;
   if (!pl.use) return ATK_OK;
@@ -480,7 +454,7 @@ int launch_chain_select(const void* cand_values, const int64_t* cand_indices, in
   int rc = ATK_ERR_DTYPE;
   ATK_DTYPE_SWITCH(dtype, E, rc = ATK_ERR_DTYPE,
                    rc = launch_chain_typed<E>(pl, cand_values, cand_indices, rows, k0, k, index_bits, values, indices,
-                                              ws, range_entries, stream));
+                                              ws, range_entries, hist_done, stream));
   return rc;
 }
 

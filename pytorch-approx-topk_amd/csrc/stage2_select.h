@@ -351,6 +351,41 @@ __device__ __forceinline__ Found find_bin_wave(const uint32_t* hist, uint32_t ne
   return f;
 }
 
+// The digit of a key when all that is known of a row's candidates is the key
+// range of every share of them (`range[0 .. entries)`: smallest and largest
+// key; shares of a superset will do): with `low` the smallest key of the row
+// and the row's keys spanning `width`, the digit is (key - low) >> shift, where
+// shift leaves the kDigitBits leading bits of the span.  (Taking the digit from
+// the offset rather than from the key's own bits keeps it fine-grained when
+// the keys straddle a power of two, where most bits of the smallest and the
+// largest key differ.)  Whole workgroup of THREADS threads; `red` is
+// 2 * THREADS / 64 words of LDS; contains a barrier, after which every thread
+// holds the result.
+template <int THREADS>
+__device__ __forceinline__ void digit_of_row(const uint2* __restrict__ range, uint32_t entries, uint32_t* red,
+                                             uint32_t& low, uint32_t& shift) {
+  constexpr int kWaves = THREADS / kWave;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  uint32_t lo = ~0u, hi = 0;
+  for (uint32_t g = tid; g < entries; g += THREADS) {
+    const uint2 r = range[g];
+    lo = r.x < lo ? r.x : lo;
+    hi = r.y > hi ? r.y : hi;
+  }
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  if (lane == 0) { red[wave] = lo; red[kWaves + wave] = hi; }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    lo = red[w] < lo ? red[w] : lo;
+    hi = red[kWaves + w] > hi ? red[kWaves + w] : hi;
+  }
+  const uint32_t span = lo >= hi ? 0u : 32u - (uint32_t)__builtin_clz(hi - lo);  // bits of the largest offset
+  low = lo >= hi ? hi : lo;
+  shift = span > (uint32_t)kDigitBits ? span - (uint32_t)kDigitBits : 0u;
+}
+
 }  // namespace regs
 
 }  // namespace select

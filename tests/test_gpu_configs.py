@@ -128,3 +128,46 @@ def test_subnormals_argmax_layouts(dtype):
         v, i = bucketed_argmax.topk_triton(x.cuda(), 96, -1, interleaved=interleaved)
         ev, ei = oracle.bucketed_argmax(x, 96, -1, interleaved=interleaved)
         assert_same(v, i, ev, ei, f"subnormals arg-max {dtype} interleaved={interleaved}")
+
+
+# ---- fp32 with two or more entries per bucket: entries are (element bits, sub-row) words ordered as doubles ----
+
+def _few_distinct_fp32(shape, seed):
+    """Rows drawn from a handful of values of both signs, zeros of both signs, subnormals, the largest
+    finite values and the infinities: every bucket is full of ties, which the lower index must win
+    under positive and negative elements alike."""
+    tiny = torch.tensor([1], dtype=torch.int32).view(torch.float32).item()          # smallest subnormal
+    pool = torch.tensor([float("-inf"), -3.4028234663852886e38, -1.5, -tiny, -0.0, 0.0, tiny, 1.5,
+                         3.4028234663852886e38, float("inf"), -1.5, -1.5, 0.0, -0.0], dtype=torch.float32)
+    g = torch.Generator().manual_seed(seed)
+    return pool[torch.randint(0, pool.numel(), shape, generator=g)]
+
+
+@pytest.mark.parametrize("j", [2, 3, 4])
+def test_fp32_ties_of_both_signs_through_every_path(j):
+    topk = _topk()
+    k = 64 * 3 * j                                   # 192 buckets
+    cases = [
+        ((6, 192 * 40), k, 1),                       # streaming kernel alone
+        ((6, 192 * 40 + 77), k, 1),                  # with a partial sub-row
+        ((300, 192 * 24), k // 2, 2),                # both stages in one kernel
+        ((2, 192 * 4096), k // 2, 2),                # slabs, merge, select
+        ((3, 48 * j * 200), 12 * j, 4),              # few buckets: folded sub-rows
+    ]
+    for shape, kk, km in cases:
+        x = _few_distinct_fp32(shape, seed=shape[1] + j)
+        v, i = topk(x.cuda(), kk, -1, j=j, k_mult=km)
+        ev, ei = oracle.topk(x, kk, -1, j=j, k_mult=km)
+        assert_same(v, i, ev, ei, f"fp32 ties j={j} shape={shape} k={kk} k_mult={km}")
+
+
+def test_fp32_negative_rows_keep_the_lower_index():
+    # all elements negative and mostly equal: the tie rule under the sign (a larger magnitude is the smaller word)
+    topk = _topk()
+    g = torch.Generator().manual_seed(11)
+    x = -torch.randint(1, 4, (5, 1 << 16), generator=g).float()
+    for j, km in [(2, 1), (4, 1), (4, 2)]:
+        k = 2048
+        v, i = topk(x.cuda(), k, -1, j=j, k_mult=km)
+        ev, ei = oracle.topk(x, k, -1, j=j, k_mult=km)
+        assert_same(v, i, ev, ei, f"negative rows j={j} k_mult={km}")
