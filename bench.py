@@ -146,23 +146,27 @@ def time_config(name: str, steps: int, warmup: int, n_inputs: int, distinct: boo
 
 
 def time_int32_indices(name: str, xs, steps: int, warmup: int):
-    """int32 against int64 indices (approx_topk.experimental.compact_indices), timed alike and
-    alternately: device microseconds per call of each, and whether the results are equal."""
+    """int32 against int64 indices, and int32 indices alone (no values written), from
+    approx_topk.experimental.compact_indices, timed alike and alternately: device microseconds
+    per call of each, and whether the results are equal."""
     import torch
 
     from approx_topk import topk
     from approx_topk.experimental.compact_indices import topk as topk_i32
+    from approx_topk.experimental.compact_indices import topk_indices
 
     rows, n, dtype, k, j, km, seed = CONFIGS[name]
-    best = {"i32": float("inf"), "i64": float("inf")}
+    best = {"i32": float("inf"), "i64": float("inf"), "only": float("inf")}
     for _ in range(3):
-        for tag, fn in (("i64", topk), ("i32", topk_i32)):
+        for tag, fn in (("i64", topk), ("i32", topk_i32), ("only", topk_indices)):
             _, dev_ms = time_steps(lambda x: fn(x, k, -1, j=j, k_mult=km), xs, steps, warmup)
             best[tag] = min(best[tag], dev_ms * 1e3 / steps)
     v32, i32 = topk_i32(xs[0], k, -1, j=j, k_mult=km)
     v64, i64 = topk(xs[0], k, -1, j=j, k_mult=km)
-    same = bool(torch.equal(i32.long(), i64) and torch.equal(v32.view(torch.uint8), v64.view(torch.uint8)))
-    return best["i32"], best["i64"], same
+    only = topk_indices(xs[0], k, -1, j=j, k_mult=km)
+    same = bool(torch.equal(i32.long(), i64) and torch.equal(v32.view(torch.uint8), v64.view(torch.uint8))
+                and torch.equal(only, i32))
+    return best["i32"], best["i64"], best["only"], same
 
 
 def parity_and_recall(name: str, x_cpu, x_gpu, sample_rows: int):
@@ -254,7 +258,7 @@ def main() -> int:
     launch_ms = dev_ms / args.steps  # device time between HIP events on the launch stream
     rec, ok, checked = parity_and_recall(name, first, xs[0], 4)
     kernels = kernels_of(name, xs[0])
-    i32_us, i64_us, i32_same = time_int32_indices(name, xs, max(50, args.steps // 2), max(20, args.warmup // 3))
+    i32_us, i64_us, only_us, i32_same = time_int32_indices(name, xs, max(50, args.steps // 2), max(20, args.warmup // 3))
     esize = in_bytes // elems
     out_bytes = rows * k * (esize + 8)
 
@@ -297,6 +301,9 @@ def main() -> int:
         "launch_us": i32_us,
         "int64_launch_us_same_loop": i64_us,
         "input_GBps": in_bytes / (i32_us * 1e-6) / 1e9,
+        # the indices alone (values == NULL in the C ABI), for consumers that only gather by them
+        "indices_only_launch_us": only_us,
+        "indices_only_input_GBps": in_bytes / (only_us * 1e-6) / 1e9,
         "equal_to_int64_result": i32_same,
     }
     del xs, first

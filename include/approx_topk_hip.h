@@ -21,7 +21,12 @@
  *   - A "row" is one slice along the top-k dimension.  Elements of a row are
  *     adjacent in memory; consecutive rows are `row_stride` elements apart.
  *   - Outputs are dense: values[rows][k] in the input dtype, indices[rows][k]
- *     as int64 positions within the row.
+ *     as int64 positions within the row.  `values` may be NULL in every entry
+ *     point that writes results: then only the indices are written, the same
+ *     ones.  (No counterpart in the reference, whose operator always returns
+ *     both, priority_queue.py:63-88: for callers that gather other tensors by
+ *     the indices and never read the selected elements; at fp32 [128, 2^20],
+ *     k = 65536, j = 2 with int32 indices the call takes 96 instead of 106 us.)
  *   - Selection order: a beats b when value(a) > value(b), or the values are
  *     equal and index(a) < index(b).  -0.0 equals +0.0, NaN ranks above +inf.
  *   - `ws` is caller-owned scratch of at least the matching *_workspace_bytes();

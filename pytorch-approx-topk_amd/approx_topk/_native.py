@@ -180,24 +180,25 @@ def _call_constants(xs: torch.Tensor, k_out: int, two_stage: bool, index_dtype: 
     return hit
 
 
-def stage1(xs: torch.Tensor, k0: int, j: int, layout: int,
-           index_dtype: torch.dtype = torch.int64) -> tuple[torch.Tensor, torch.Tensor]:
+def stage1(xs: torch.Tensor, k0: int, j: int, layout: int, index_dtype: torch.dtype = torch.int64,
+           want_values: bool = True) -> tuple[torch.Tensor | None, torch.Tensor]:
     """Per-bucket top-j along the last dim: (values[..., k0], indices[..., k0]).
 
-    ``index_dtype``: torch.int64 (the operator's contract) or torch.int32."""
+    ``index_dtype``: torch.int64 (the operator's contract) or torch.int32.
+    ``want_values=False``: only the indices are written; values is None."""
     require_gpu(xs)
     step = None
     if not xs.is_contiguous():
         xs, _, _, step = rows_view(xs)
     rows, n, code, shape, entry = _call_constants(xs, k0, False, index_dtype)
     device = xs.device
-    values = torch.empty(shape, dtype=xs.dtype, device=device)
+    values = torch.empty(shape, dtype=xs.dtype, device=device) if want_values else None
     indices = torch.empty(shape, dtype=index_dtype, device=device)
     with _on_device(device):
         need = _stage1_workspace(rows, n, k0, j, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
         status = entry(xs.data_ptr(), rows, n, n if step is None else step, k0, j, layout, code,
-                       values.data_ptr(), indices.data_ptr(),
+                       values.data_ptr() if want_values else None, indices.data_ptr(),
                        ws.data_ptr() if ws is not None else None, need, _stream(device))
     if status != 0:
         check(status)
@@ -225,8 +226,8 @@ def select(cand_values: torch.Tensor, cand_indices: torch.Tensor, k: int,
     return values, indices
 
 
-def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int,
-         index_dtype: torch.dtype = torch.int64) -> tuple[torch.Tensor, torch.Tensor]:
+def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int, index_dtype: torch.dtype = torch.int64,
+         want_values: bool = True) -> tuple[torch.Tensor | None, torch.Tensor]:
     """Stage 1 (k0 candidates) and stage 2 (k survivors) along the last dim."""
     require_gpu(xs)
     step = None
@@ -234,14 +235,14 @@ def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int,
         xs, _, _, step = rows_view(xs)
     rows, n, code, shape, entry = _call_constants(xs, k, True, index_dtype)
     device = xs.device
-    values = torch.empty(shape, dtype=xs.dtype, device=device)
+    values = torch.empty(shape, dtype=xs.dtype, device=device) if want_values else None
     indices = torch.empty(shape, dtype=index_dtype, device=device)
     with _on_device(device):
         pitch = n if step is None else step
         need = _topk_workspace(xs.data_ptr() % 16, rows, n, pitch, k0, j, k, layout, code)
         ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
         status = entry(xs.data_ptr(), rows, n, pitch, k0, j, k, layout, code,
-                       values.data_ptr(), indices.data_ptr(),
+                       values.data_ptr() if want_values else None, indices.data_ptr(),
                        ws.data_ptr() if ws is not None else None, need, _stream(device))
     if status != 0:
         check(status)

@@ -47,7 +47,8 @@ def _topk(
     interleaved: bool = True,
     multithread_buckets: bool | None = False,
     index_dtype: torch.dtype = torch.int64,
-) -> tuple[Tensor, Tensor]:
+    want_values: bool = True,
+) -> tuple[Tensor | None, Tensor]:
     """Approximate top-``k`` of ``xs`` along ``dim``.
 
     The slice is cut into ``b = k_mult * k / j`` buckets (interleaved: bucket
@@ -77,7 +78,7 @@ def _topk(
 
     if k0 == 0:
         values, indices = _empty_result(xs, 0, dim)
-        return values, indices.to(index_dtype)
+        return (values if want_values else None), indices.to(index_dtype)
     if j < 1 or j > 4:
         raise RuntimeError("topk: j must 0 < j < 5")
     if k0 % j != 0:
@@ -89,25 +90,25 @@ def _topk(
     layout = _native.INTERLEAVED if interleaved else _native.BALANCED
     if dim == last and n != 0 and xs.ndim and xs.numel():  # the common case, straight through
         if k_mult == 1:
-            return _native.stage1(xs, k0, j, layout, index_dtype)
-        return _native.topk(xs, k0, j, k, layout, index_dtype)
+            return _native.stage1(xs, k0, j, layout, index_dtype, want_values)
+        return _native.topk(xs, k0, j, k, layout, index_dtype, want_values)
     if xs.numel() == 0:
         values, indices = _empty_result(xs, k, dim)
-        return values, indices.to(index_dtype)
+        return (values if want_values else None), indices.to(index_dtype)
 
     rows = xs if xs.ndim else xs.reshape(1)
     moved = dim != last and xs.ndim > 1
     if moved:
         rows = rows.movedim(dim, -1)
     if k_mult == 1:
-        values, indices = _native.stage1(rows, k0, j, layout, index_dtype)
+        values, indices = _native.stage1(rows, k0, j, layout, index_dtype, want_values)
     else:
-        values, indices = _native.topk(rows, k0, j, k, layout, index_dtype)
+        values, indices = _native.topk(rows, k0, j, k, layout, index_dtype, want_values)
     if moved:
-        values = values.movedim(-1, dim).contiguous()
+        values = values.movedim(-1, dim).contiguous() if want_values else None
         indices = indices.movedim(-1, dim).contiguous()
     if not xs.ndim:
-        values, indices = values.reshape(()), indices.reshape(())
+        values, indices = (values.reshape(()) if want_values else None), indices.reshape(())
     return values, indices
 
 

@@ -60,7 +60,7 @@ int check_stage1(const void* x, int64_t rows, int64_t n, int64_t row_stride, int
   const bool padded = layout == ATK_CEIL_CHUNK || layout == ATK_INTERLEAVED_PADDED;
   if (padded && j != 1) return ATK_ERR_LAYOUT;
   if (padded ? n < 1 : k0 > n) return ATK_ERR_K;
-  if (!x || !values || !indices || row_stride < n) return ATK_ERR_ARG;
+  if (!x || !indices || row_stride < n) return ATK_ERR_ARG;  // (values may be NULL: indices only)
   return ATK_OK;
 }
 
@@ -228,7 +228,7 @@ int atk_select(const void* cand_values, const int64_t* cand_indices, int64_t row
   if (atk::elem_bytes(dtype) == 0) return ATK_ERR_DTYPE;
   if (rows < 0 || k0 < 0 || k < 0 || k > k0 || index_bound < 0) return ATK_ERR_K;
   if (rows == 0 || k == 0) return ATK_OK;
-  if (!cand_values || !cand_indices || !values || !indices) return ATK_ERR_ARG;
+  if (!cand_values || !cand_indices || !indices) return ATK_ERR_ARG;  // (values may be NULL: indices only)
   if (!aligned_to(cand_indices, 8)) return ATK_ERR_ALIGN;
   if (const int rca = check_alignment(cand_values, values, dtype, atk::IndexOut{indices, 0}, ws); rca != ATK_OK)
     return rca;

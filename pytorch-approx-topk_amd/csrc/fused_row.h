@@ -86,7 +86,7 @@ __device__ __forceinline__ void select_from_lds(Sh& sh, const typename E::raw_t*
         return Got{index, value};
       },
       [&](uint32_t, uint32_t o, const Got& got) {
-        ov[o] = got.value;
+        if (values != nullptr) ov[o] = got.value;
         indices.put(oi + o, got.index);
       });
 }
@@ -446,7 +446,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
           index[1] = result(make_uint2(e01.z, e01.w), pv.e[1]);
           index[2] = result(make_uint2(e23.x, e23.y), pv.e[2]);
           index[3] = result(make_uint2(e23.z, e23.w), pv.e[3]);
-          *reinterpret_cast<stream::Pack<raw_t, 4>*>(ov + at) = pv;
+          if (values != nullptr) *reinterpret_cast<stream::Pack<raw_t, 4>*>(ov + at) = pv;
           if (indices.narrow) {
             stream::Pack<int32_t, 4> pi;
 #pragma unroll
@@ -465,7 +465,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
         for (uint32_t at = tid; at < k; at += nt) {
           raw_t value;
           const uint32_t index = result(stage[at], value);
-          ov[at] = value;
+          if (values != nullptr) ov[at] = value;
           indices.put(oi + at, (int64_t)index);
         }
       }
@@ -476,7 +476,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
   ATK_STATIC_FOR(e, NC) {
     if ((selected >> e) & 1u) {
       if (o < k) {
-        ov[o] = queue.template raw<e / J, e % J>();
+        if (values != nullptr) ov[o] = queue.template raw<e / J, e % J>();
         indices.put(oi + o, (int64_t)index_of(std::integral_constant<int, e>{}));
       }
       ++o;

@@ -237,7 +237,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
       const int64_t o = (row * g.b + c) * J;
       ATK_STATIC_FOR(sl, J) {
         const uint32_t p = M::pos(acc[N - J + sl]);
-        values[o + sl] = (int64_t)p < g.n ? stream::element_of<E>(acc[N - J + sl], xr, p) : E::pad_raw;
+        if (values != nullptr) values[o + sl] = (int64_t)p < g.n ? stream::element_of<E>(acc[N - J + sl], xr, p) : E::pad_raw;
         indices.put(o + sl, p);
       } ATK_STATIC_END;
     }
@@ -294,7 +294,7 @@ __global__ __launch_bounds__(64) void contig_merge_kernel(const typename E::raw_
   const int64_t o = (row * g.b + c) * J;
   ATK_STATIC_FOR(sl, J) {
     const uint32_t p = M::pos(acc[N - J + sl]);
-    values[o + sl] = (int64_t)p < g.n ? stream::element_of<E>(acc[N - J + sl], xr, p) : E::pad_raw;
+    if (values != nullptr) values[o + sl] = (int64_t)p < g.n ? stream::element_of<E>(acc[N - J + sl], xr, p) : E::pad_raw;
     indices.put(o + sl, p);
   } ATK_STATIC_END;
 }

@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void stage1_lane_per_bucket_kernel(
 #pragma unroll
   for (int s = 0; s < J; ++s) {
     const int64_t p = pos[s];
-    values[out + s] = (p >= 0 && p < n) ? xr[p] : E::pad_raw;
+    if (values != nullptr) values[out + s] = (p >= 0 && p < n) ? xr[p] : E::pad_raw;
     indices.put(out + s, p);
   }
 }

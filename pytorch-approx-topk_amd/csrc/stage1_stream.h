@@ -732,11 +732,13 @@ __device__ __forceinline__ void emit(const Geom& g, const Sink<typename E::raw_t
     if constexpr (V > 1) {
       // V*J values = J stores of V elements; V*J int64 = V*J/2 16-byte stores
       // (int32: 16-byte stores when V*J is a multiple of 4, else 8-byte ones)
-      ATK_STATIC_FOR(t, J) {
-        Pack<raw_t, V> pv;
-        ATK_STATIC_FOR(e, V) { pv.e[e] = queue.template raw<(t * V + e) / J, (t * V + e) % J>(); } ATK_STATIC_END;
-        reinterpret_cast<Pack<raw_t, V>*>(ov)[t] = pv;
-      } ATK_STATIC_END;
+      if (out.values != nullptr) {
+        ATK_STATIC_FOR(t, J) {
+          Pack<raw_t, V> pv;
+          ATK_STATIC_FOR(e, V) { pv.e[e] = queue.template raw<(t * V + e) / J, (t * V + e) % J>(); } ATK_STATIC_END;
+          reinterpret_cast<Pack<raw_t, V>*>(ov)[t] = pv;
+        } ATK_STATIC_END;
+      }
       if (out.indices.narrow) {
         constexpr int kPer = (V * J) % 4 == 0 ? 4 : 2;
         int32_t* oi = static_cast<int32_t*>(out.indices.base) + o;
@@ -761,7 +763,7 @@ __device__ __forceinline__ void emit(const Geom& g, const Sink<typename E::raw_t
       }
     } else {
       ATK_STATIC_FOR(sl, J) {
-        ov[sl] = queue.template raw<0, sl>();
+        if (out.values != nullptr) ov[sl] = queue.template raw<0, sl>();
         out.indices.put(o + sl, col + (int64_t)queue.template position<0, sl>() * g.b);
       } ATK_STATIC_END;
     }
@@ -806,7 +808,10 @@ __device__ __forceinline__ void exact_columns(const typename E::raw_t* __restric
     if (out.part_values == nullptr) {
       const int64_t o = (row * g.b + c) * J;
 #pragma unroll
-      for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices.put(o + s, c + (int64_t)pos[s] * g.b); }
+      for (int s = 0; s < J; ++s) {
+        if (out.values != nullptr) out.values[o + s] = val[s];
+        out.indices.put(o + s, c + (int64_t)pos[s] * g.b);
+      }
     } else {
       const int64_t o = ((row * g.slabs + slab) * g.b + c) * J;
 #pragma unroll
@@ -1117,7 +1122,7 @@ __device__ __forceinline__ void fold_columns(const typename E::raw_t* __restrict
         const typename E::raw_t value = element_of<E>(acc[N - J + sl], xr, index);
         if (out.part_values == nullptr) {
           const int64_t o = (row * b + c) * J + sl;
-          out.values[o] = value;
+          if (out.values != nullptr) out.values[o] = value;
           out.indices.put(o, index);
         } else {
           const int64_t o = ((row * g.slabs + slab) * b + c) * J + sl;
@@ -1154,7 +1159,10 @@ __device__ __forceinline__ void fold_columns_exact(const typename E::raw_t* __re
     if (out.part_values == nullptr) {
       const int64_t o = (row * b + c) * J;
 #pragma unroll
-      for (int s = 0; s < J; ++s) { out.values[o + s] = val[s]; out.indices.put(o + s, c + (int64_t)pos[s] * b); }
+      for (int s = 0; s < J; ++s) {
+        if (out.values != nullptr) out.values[o + s] = val[s];
+        out.indices.put(o + s, c + (int64_t)pos[s] * b);
+      }
     } else {
       const int64_t o = ((row * g.slabs + slab) * b + c) * J;
 #pragma unroll
@@ -1325,7 +1333,7 @@ __global__ __launch_bounds__(kMergeThreads) void stream_merge_kernel(
     const int64_t o = (row * b + c) * J;
     ATK_STATIC_FOR(s, J) {
       const int64_t index = c + (int64_t)M::pos(acc[N - J + s]) * b;
-      values[o + s] = element_of<E>(acc[N - J + s], xr, index);
+      if (values != nullptr) values[o + s] = element_of<E>(acc[N - J + s], xr, index);
       indices.put(o + s, index);
     } ATK_STATIC_END;
   }

@@ -249,7 +249,10 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
     const int64_t out_first = (int64_t)row * k;
     select::compact(
         sh, k0, k, survives, [&](uint32_t i) { return Candidate{rv[i], ri[i]}; },
-        [&](uint32_t, uint32_t o, const Candidate& c) { out_values[o] = c.value; indices.put(out_first + o, c.index); });
+        [&](uint32_t, uint32_t o, const Candidate& c) {
+          if (values != nullptr) out_values[o] = c.value;
+          indices.put(out_first + o, c.index);
+        });
     return;
   }
   const bool cut_digit = s.need != s.count;  // else every member of B survives
@@ -335,7 +338,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
     if (sel[u]) {
       const uint32_t at = o + select::rank_in(m);
       if (at < k) {
-        ov[at] = raw[u];
+        if (values != nullptr) ov[at] = raw[u];
         indices.put(oi + at, (int64_t)(uint32_t)~inv[u]);
       }
     }

@@ -293,7 +293,7 @@ __global__ __launch_bounds__(kThreads) void ms_emit_kernel(
       [&](uint32_t i) { return Candidate<raw_t>{cv[i], ci[i]}; },
       [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) {
         if (first + o < k) {  // always true for consistent inputs; keeps a wrong cut from writing out of bounds
-          ov[first + o] = c.value;
+          if (values != nullptr) ov[first + o] = c.value;
           indices.put(oi + first + o, c.index);
         }
       });

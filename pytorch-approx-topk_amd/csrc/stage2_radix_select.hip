@@ -85,7 +85,10 @@ __global__ __launch_bounds__(COPIES == 8 ? 1024 : 256) void select_kernel(
   select::compact(
       sh, k0, k, survives,
       [&](uint32_t i) { return Candidate<raw_t>{cv[i], ci[i]}; },
-      [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) { ov[o] = c.value; indices.put(oi + o, c.index); });
+      [&](uint32_t, uint32_t o, const Candidate<raw_t>& c) {
+        if (values != nullptr) ov[o] = c.value;
+        indices.put(oi + o, c.index);
+      });
 }
 
 // LDS a workgroup may use for keys; the rest of the 160 KB of a gfx950 CU is
