@@ -599,9 +599,14 @@ template <typename E, int J, int V> struct WideQueue {
     const uint32_t lo = np ^ (uint32_t)((int32_t)hi >> 31);
     return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
   }
-  __device__ static __forceinline__ void insert(double (&col)[J], double w) {
-    ATK_STATIC_FOR(s, J - 1) { col[s] = max_f64(col[s], min_f64(w, col[s + 1])); } ATK_STATIC_END;
-    col[J - 1] = max_f64(col[J - 1], w);
+  // FILLED: entries the column is known to hold already (its last ones; the others are empty)
+  template <int FILLED = J> __device__ static __forceinline__ void insert(double (&col)[J], double w) {
+    ATK_STATIC_FOR(s, J - 1) {
+      if constexpr (s + 1 + FILLED == J) col[s] = min_f64(w, col[s + 1]);
+      else if constexpr (s + 1 + FILLED > J) col[s] = max_f64(col[s], min_f64(w, col[s + 1]));
+    } ATK_STATIC_END;
+    if constexpr (FILLED == 0) col[J - 1] = w;
+    else col[J - 1] = max_f64(col[J - 1], w);
   }
 
   __device__ __forceinline__ void reset() {
@@ -618,7 +623,7 @@ template <typename E, int J, int V> struct WideQueue {
     ATK_STATIC_FOR(v, V) { c[v] = __uint_as_float(pk.e[v]) + 0.0f; } ATK_STATIC_END;
     ATK_STATIC_FOR(h, V / 2) { nan_mask |= __ballot(__builtin_isunordered(c[2 * h], c[2 * h + 1])); } ATK_STATIC_END;
     if constexpr (V % 2 != 0) nan_mask |= __ballot(__builtin_isunordered(c[V - 1], c[V - 1]));
-    ATK_STATIC_FOR(v, V) { insert(q[v], word(c[v], np)); } ATK_STATIC_END;
+    ATK_STATIC_FOR(v, V) { insert<FILLED>(q[v], word(c[v], np)); } ATK_STATIC_END;
   }
   template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
     const float c = __uint_as_float(raw) + 0.0f;
