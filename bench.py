@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # the kernels the planner reports for the call: a change of plan leaves the figure out (null)
 # rather than stale.  Source: profiles/stream_kernel_f32_j2_c2_hbm_traffic.md.
 MEASURED_TRAFFIC_BYTES = {
-    "stream_kernel<f32, J=2, V=4, W=8, U=8, RUN=4, PACKED=0> grid=16384 block=512 fold=1 slabs=1": 637_602_610,
+    "stream_kernel<f32, J=2, V=4, W=8, U=8, RUN=4, PACKED=0> grid=16384 block=512 fold=1 slabs=1": 637_658_986,
 }
 
 # name -> (rows, n, dtype, k, j, k_mult, seed)
@@ -264,6 +264,9 @@ def main() -> int:
     ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--all-configs", action="store_true", help="accepted for compatibility: the default now")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-index-variants", action="store_true",
+                    help="skip the int32-index and indices-only timings (they launch the same kernel "
+                         "with less output, which blurs per-kernel profiles of the workload)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 512 MiB device copy a few times (a kernel of known traffic for "
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -291,7 +294,9 @@ def main() -> int:
     launch_ms = dev_ms / args.steps  # device time between HIP events on the launch stream
     rec, ok, checked = parity_and_recall(name, first, xs[0], 4)
     kernels = kernels_of(name, xs[0])
-    i32_us, i64_us, only_us, i32_same = time_int32_indices(name, xs, max(50, args.steps // 2), max(20, args.warmup // 3))
+    if not args.no_index_variants:
+        i32_us, i64_us, only_us, i32_same = time_int32_indices(name, xs, max(50, args.steps // 2),
+                                                               max(20, args.warmup // 3))
     esize = in_bytes // elems
     out_bytes = rows * k * (esize + 8)
 
@@ -330,15 +335,16 @@ def main() -> int:
     }
     # not the metric: the operator's contract is int64 indices; shown because the index write is
     # part of what keeps this shape from the read-only rate
-    result["int32_indices"] = {
-        "launch_us": i32_us,
-        "int64_launch_us_same_loop": i64_us,
-        "input_GBps": in_bytes / (i32_us * 1e-6) / 1e9,
-        # the indices alone (values == NULL in the C ABI), for consumers that only gather by them
-        "indices_only_launch_us": only_us,
-        "indices_only_input_GBps": in_bytes / (only_us * 1e-6) / 1e9,
-        "equal_to_int64_result": i32_same,
-    }
+    if not args.no_index_variants:
+        result["int32_indices"] = {
+            "launch_us": i32_us,
+            "int64_launch_us_same_loop": i64_us,
+            "input_GBps": in_bytes / (i32_us * 1e-6) / 1e9,
+            # the indices alone (values == NULL in the C ABI), for consumers that only gather by them
+            "indices_only_launch_us": only_us,
+            "indices_only_input_GBps": in_bytes / (only_us * 1e-6) / 1e9,
+            "equal_to_int64_result": i32_same,
+        }
     del xs, first
     torch.cuda.empty_cache()
 
