@@ -23,9 +23,10 @@ int launch_stage1_lane_per_bucket(const void* x, int64_t rows, int64_t n,
 // order key of shares of every row's candidates (shares of a superset of them
 // will do: the ranges only say which key bits all candidates have in common),
 // that select's row states cleared, and its histogram either cleared or
-// already filled with the candidates' digits.  The stage-1 launcher sets
-// `entries`: shares per row it wrote (0: it wrote nothing and cleared nothing),
-// and `hist_done`: the histogram holds the candidates' digits.
+// already filled with the candidates' digits (`want_hist`, set by the select's
+// side: whether it has a use for that).  The stage-1 launcher sets `entries`:
+// shares per row it wrote (0: it wrote nothing and cleared nothing), and
+// `hist_done`: the histogram holds the candidates' digits.
 struct KeyRangeOut {
   uint2* range;             // [rows][entries]
   uint32_t capacity;        // entries per row that fit
@@ -33,6 +34,7 @@ struct KeyRangeOut {
   uint32_t hist_words;
   uint32_t* state;          // [rows][state_words]
   uint32_t state_words;
+  uint32_t want_hist;
   uint32_t entries;
   uint32_t hist_done;
 };

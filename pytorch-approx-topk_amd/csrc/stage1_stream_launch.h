@@ -60,13 +60,16 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
   constexpr int VF = full_vec((int)sizeof(raw_t));
   // Kernels that end in the merge of slabs can leave a chained select its key
   // ranges (one per scanning workgroup) and its histogram.
-  KeyRangeOut left{};
+  KeyRangeOut left{}, left_to_merge{};
   const int64_t scan_blocks = (int64_t)pl.slabs * pl.col_tiles;  // per row
   if (ranges != nullptr && ranges->range != nullptr && E::key_bits <= 32 && pl.merge &&
       scan_blocks <= (int64_t)ranges->capacity) {
     ranges->entries = (uint32_t)scan_blocks;
-    ranges->hist_done = 1;
     left = *ranges;
+    if (ranges->want_hist != 0) {
+      ranges->hist_done = 1;
+      left_to_merge = left;
+    }
   }
   const int rc = pl.vec > 1 ? launch_w<E, J, VF>(pl, x, out, g, rows, stream, left)
                             : launch_w<E, J, 1>(pl, x, out, g, rows, stream, left);
@@ -81,7 +84,7 @@ static int launch_j(const Plan& pl, const typename E::raw_t* x, const Sink<typen
   hipLaunchKernelGGL((stream_merge_kernel<E, J>), dim3((unsigned)(blocks_per_row * rows)),
                      dim3(kMergeThreads), 0,
                      stream, x, g.row_stride, (const raw_t*)out.part_values, (const uint32_t*)out.part_pos,
-                     b, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices, left);
+                     b, pl.slabs, cb, (uint32_t)blocks_per_row, out.values, out.indices, left_to_merge);
   return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
 }
 

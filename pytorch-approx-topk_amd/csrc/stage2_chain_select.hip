@@ -62,6 +62,7 @@ constexpr uint32_t kRangeCapacity = 4096;
 
 struct ChainPlan {
   bool use;
+  bool solo;        // one launch does it (chain_solo_kernel)
   uint32_t groups;  // workgroups per row
   uint32_t range_capacity;
   size_t range_off, hist_off, state_off, above_off, list_word_off, list_at_off, total;
@@ -347,6 +348,185 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// The chain in one launch, for rows of up to kSoloMaxCandidates candidates.
+//
+// The launches of the chain cost more than their work (4-7 us each against
+// 1-2 us), so for rows short enough every workgroup does the row-wide steps
+// itself, redundantly, and only its own segment's write-out is its own: it
+// reads all of the row's keys into registers (k0 / 1024 per thread: candidate
+// u * 1024 + t is thread t's u-th, so that a thread's u-th key belongs to
+// segment u), builds the digit histogram in LDS, finds the digit B of the k-th
+// best, lists the members of B in LDS and ranks them, counts the survivors of
+// the segments before its own from the keys it holds, and writes its segment.
+// The row's keys are read groups-times over (32 x 128 KiB at fp32 [1, 32768]),
+// from L2 for the most part.  The key ranges come from stage 1 or from a
+// chain_range_kernel launch, as before.
+// ---------------------------------------------------------------------------
+constexpr int kSoloThreads = 1024;  // == kSegment
+constexpr int kSoloWaves = kSoloThreads / select::kWave;
+constexpr uint32_t kSoloRankDirect = 512;
+static_assert((uint32_t)kSoloThreads == kSegment, "a thread's u-th candidate lies in segment u");
+
+template <typename E, int NPT>
+__global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
+    const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
+    uint32_t k, uint32_t groups, int index_bits, const uint2* __restrict__ range, uint32_t entries,
+    typename E::raw_t* __restrict__ values, const IndexOut indices) {
+  using raw_t = typename E::raw_t;
+  using key_t = typename E::key_t;
+  extern __shared__ __align__(16) unsigned char dyn_lds[];
+  __shared__ __align__(16) uint32_t hist[regs::kHistWords];
+  __shared__ select::SharedT<2> sh;
+  __shared__ regs::Found found;
+  __shared__ uint32_t red[2 * kSoloWaves];
+  __shared__ uint32_t wave_before[kSoloWaves], wave_kept[kSoloWaves];
+  __shared__ uint32_t list_count;
+  __shared__ uint64_t cut_word;
+  uint64_t* words = reinterpret_cast<uint64_t*>(dyn_lds);
+  uint32_t* ats = reinterpret_cast<uint32_t*>(dyn_lds + (size_t)(kListCap + 8) * sizeof(uint64_t));
+  const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
+  const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
+  const raw_t* cv = cand_values + (int64_t)row * k0;
+  const int64_t* ci = cand_indices + (int64_t)row * k0;
+
+  // (the key ranges are asked for first, so that they travel with the keys)
+  const uint2 folded = regs::fold_ranges<kSoloThreads>(range + (size_t)row * entries, entries);
+  // all keys of the row, NPT per thread (0 past the row's end; `valid` says so)
+  uint32_t key[NPT];
+  auto valid = [&](int u) -> bool { return (uint32_t)u * kSoloThreads + tid < k0; };
+  {
+    raw_t raw[NPT];
+#pragma unroll
+    for (int u = 0; u < NPT; ++u) raw[u] = valid(u) ? cv[(uint32_t)u * kSoloThreads + tid] : (raw_t)0;
+#pragma unroll
+    for (int u = 0; u < NPT; ++u) key[u] = (uint32_t)E::key(raw[u]);
+  }
+  for (uint32_t i = tid; i < (uint32_t)regs::kHistWords; i += kSoloThreads) hist[i] = 0;
+  if (tid == 0) { list_count = 0; cut_word = 0; }
+  uint32_t low, shift;
+  regs::digit_from_folded<kSoloThreads>(folded, red, low, shift);  // (its barrier covers the clearing)
+#pragma unroll
+  for (int u = 0; u < NPT; ++u)
+    if (valid(u)) atomicAdd(&hist[regs::hist_slot((key[u] - low) >> shift)], 1u);
+  __syncthreads();
+  if (wave == 0) {
+    const regs::Found f = regs::find_bin_wave(hist, k, k0, lane);
+    if (lane == 0) found = f;
+  }
+  __syncthreads();
+  const regs::Found f = found;
+  const bool cut_digit = f.need != f.count;  // else every member of B survives
+  if (cut_digit && f.count > kListCap) {
+    // The cut digit holds more candidates than the list: the row's first
+    // workgroup runs the block-wide radix select of stage2_select.h over all of
+    // the row's candidates, read from global memory (slow, but only rows with
+    // thousands of equal keys around the cut come here).
+    if (g != 0) return;
+    auto key_at = [&](uint32_t i) -> key_t { return E::key(cv[i]); };
+    auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)ci[i]; };
+    const select::Cut<key_t> whole = select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
+    auto survives = [&](uint32_t i) -> bool {
+      const key_t kk = key_at(i);
+      if (kk != whole.T) return kk > whole.T;
+      return whole.index_cut == ~0ull || index_at(i) <= whole.index_cut;
+    };
+    struct Candidate { raw_t value; int64_t index; };
+    raw_t* out_values = values + (int64_t)row * k;
+    const int64_t out_first = (int64_t)row * k;
+    select::compact(
+        sh, k0, k, survives, [&](uint32_t i) { return Candidate{cv[i], ci[i]}; },
+        [&](uint32_t, uint32_t o, const Candidate& c) {
+          if (values != nullptr) out_values[o] = c.value;
+          indices.put(out_first + o, c.index);
+        });
+    return;
+  }
+  // this thread's candidate of segment g (asked for here and not with the keys:
+  // measured, the index load up there makes the kernel 5 us slower)
+  const uint32_t own = g * kSoloThreads + tid;
+  const bool own_valid = own < k0;
+  const raw_t own_raw = own_valid ? cv[own] : (raw_t)0;
+  const uint32_t own_inv = own_valid ? ~(uint32_t)ci[own] : 0u;
+  // survivors above the cut digit (or in it, when it belongs whole) in the
+  // segments before this one, and the members of a cut digit listed
+  uint32_t before = 0;
+  uint32_t own_key = 0;
+#pragma unroll
+  for (int u = 0; u < NPT; ++u) {
+    const uint32_t d = (key[u] - low) >> shift;
+    const bool ok = valid(u);
+    if ((uint32_t)u < g) before += (ok && (d > f.digit || (d == f.digit && !cut_digit))) ? 1u : 0u;
+    if ((uint32_t)u == g) own_key = key[u];
+    if (ok && cut_digit && d == f.digit) {
+      const uint32_t at = (uint32_t)u * kSoloThreads + tid;
+      const uint32_t slot = atomicAdd(&list_count, 1u);
+      words[slot] = (uint64_t)key[u] << 32;  // (the index follows below, for all members in one trip to memory)
+      ats[slot] = at;
+    }
+  }
+  const uint32_t n = cut_digit ? f.count : 0u;  // (== list_count after the barrier)
+  if (tid < 8u) {  // entries past the list's end beat nothing (ranking reads it in groups of eight)
+    words[n + tid] = 0ull;
+    ats[n + tid] = ~0u;
+  }
+  __syncthreads();
+  uint64_t cut = 0;  // the weakest surviving member of B (0: all of them survive)
+  if (n != 0) {
+    for (uint32_t i = tid; i < n; i += kSoloThreads) words[i] |= (uint64_t)(~(uint32_t)ci[ats[i]]);
+    __syncthreads();
+    if (n <= kSoloRankDirect) {
+      if (tid < n) {  // thread t counts the entries better than entry t: the need-th best is the cut
+        const uint64_t mine = words[tid];
+        uint32_t better = 0;
+        for (uint32_t m = 0; m < n; m += 8) {
+          uint64_t got[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) got[e] = words[m + e];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) better += got[e] > mine ? 1u : 0u;
+        }
+        if (better + 1 == f.need) cut_word = mine;
+      }
+      __syncthreads();
+      cut = cut_word;
+    } else {  // a longer list: the block-wide radix select over its words (all distinct)
+      auto key_at = [&](uint32_t i) -> uint64_t { return words[i]; };
+      auto index_at = [&](uint32_t) -> uint64_t { return 0; };
+      cut = select::find_cut<uint64_t, 64>(sh, n, f.need, 1, key_at, index_at).T;
+    }
+    for (uint32_t i = tid; i < n; i += kSoloThreads) before += (ats[i] < g * kSoloThreads && words[i] >= cut) ? 1u : 0u;
+  }
+  // this thread's own candidate
+  const uint32_t own_d = (own_key - low) >> shift;
+  const bool sel = own_valid && (own_d > f.digit ||
+                                 (own_d == f.digit && (((uint64_t)own_key << 32) | own_inv) >= cut));
+  const uint64_t m = __ballot(sel);
+  before = regs::wave_scan(before);
+  if (lane == select::kWave - 1) wave_before[wave] = before;
+  if (lane == 0) wave_kept[wave] = (uint32_t)__popcll(m);
+  __syncthreads();
+  uint32_t at = 0;
+#pragma unroll
+  for (int w = 0; w < kSoloWaves; ++w) {
+    at += wave_before[w];
+    if ((uint32_t)w < wave) at += wave_kept[w];
+  }
+  if (sel) {
+    at += select::rank_in(m);
+    if (at < k) {
+      if (values != nullptr) values[(int64_t)row * k + at] = own_raw;
+      indices.put((int64_t)row * k + at, (int64_t)(uint32_t)~own_inv);
+    }
+  }
+}
+
+// Rows the one-launch form takes: short enough for the keys to sit in registers
+// and for the redundant reads (every workgroup reads the whole row) to stay small.
+constexpr int64_t kSoloMaxCandidates = 64 * kSoloThreads;
+constexpr int64_t kSoloMaxRedundantBytes = 32ll << 20;
+
 // Rows for which the chain beats one workgroup per row: few rows (one workgroup
 // per row already fills the GPU with many), enough candidates that a single CU
 // is what bounds them, keys of at most 32 bits and indices below 2^31.
@@ -361,6 +541,7 @@ ChainPlan plan_chain(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, i
   if (es == 0 || es > 4 || rows <= 0 || rows > kChainMaxRows || k <= 0 || k >= k0) return pl;
   if (k0 < kChainMinCandidates || k0 > kChainMaxCandidates || index_bound > 0x7fffffffll) return pl;
   pl.groups = (uint32_t)((k0 + kSegment - 1) / kSegment);
+  pl.solo = k0 <= kSoloMaxCandidates && rows * (int64_t)pl.groups * k0 * es <= kSoloMaxRedundantBytes;
   pl.range_off = 0;
   pl.range_capacity = pl.groups > kRangeCapacity ? pl.groups : kRangeCapacity;
   pl.hist_off = align_up((size_t)rows * pl.range_capacity * sizeof(uint2), 256);
@@ -395,6 +576,20 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
                          state);
       entries = pl.groups;
     }
+    if (pl.solo) {
+      const size_t solo_lds = (size_t)(kListCap + 8) * (sizeof(uint64_t) + sizeof(uint32_t));
+      const dim3 solo_block(kSoloThreads);
+      raw_t* out = static_cast<raw_t*>(values);
+#define ATK_SOLO(NPT)                                                                                            \
+  hipLaunchKernelGGL((chain_solo_kernel<E, NPT>), grid, solo_block, solo_lds, stream, cv, cand_indices,          \
+                     (uint32_t)k0, (uint32_t)k, pl.groups, index_bits, (const uint2*)range, entries, out, indices)
+      if (k0 <= 8 * kSoloThreads) ATK_SOLO(8);
+      else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16);
+      else if (k0 <= 32 * kSoloThreads) ATK_SOLO(32);
+      else ATK_SOLO(64);
+#undef ATK_SOLO
+      return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+    }
     if (!hist_done || range_entries == 0)
       hipLaunchKernelGGL((chain_hist_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups,
                          (const uint2*)range, entries, hist);
@@ -423,6 +618,11 @@ bool describe_chain_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bo
   const ChainPlan pl = plan_chain(rows, k0, k, index_bound, dtype);
   if (!pl.use) return false;
   const std::string t = dtype_name(dtype);
+  if (pl.solo) {
+    out += "[chain_range_kernel<" + t + "> unless stage 1 left key ranges] + chain_solo_kernel<" + t + "> grid=" +
+           std::to_string(rows * (int64_t)pl.groups) + " block=" + std::to_string(kSoloThreads);
+    return true;
+  }
   out += "[chain_range_kernel<" + t + "> + chain_hist_kernel<" + t +
          "> unless stage 1 left key ranges and histogram] + chain_refine_kernel<" + t +
          "> + chain_emit_kernel<" + t + "> grid=" + std::to_string(rows * (int64_t)pl.groups) + " block=" +
@@ -442,6 +642,7 @@ KeyRangeOut chain_select_ranges(int64_t rows, int64_t k0, int64_t k, int64_t ind
   out.hist_words = regs::kHistWords;
   out.state = reinterpret_cast<uint32_t*>(base + pl.state_off);
   out.state_words = (uint32_t)(sizeof(RowState) / sizeof(uint32_t));
+  out.want_hist = pl.solo ? 0u : 1u;
   return out;
 }
 

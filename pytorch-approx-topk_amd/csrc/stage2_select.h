@@ -301,22 +301,30 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
   return v;
 }
 
-// Smallest and largest of a 32-bit value over the 64 lanes of a wave, in every lane.
+// Smallest and largest of a 32-bit value over the 64 lanes of a wave, in every
+// lane: the steps of wave_scan with min / max in place of the sum (lanes without
+// a source take the identity), then the last lane's result for all.
 __device__ __forceinline__ uint32_t wave_min(uint32_t v) {
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const uint32_t other = (uint32_t)__shfl_xor((int)v, d, kWave);
-    v = other < v ? other : v;
+#define ATK_WAVE_STEP(ctrl, rows)                                                                      \
+  {                                                                                                     \
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)~0u, (int)v, ctrl, rows, 0xf, false); \
+    v = o < v ? o : v;                                                                                  \
   }
-  return v;
+  ATK_WAVE_STEP(0x111, 0xf) ATK_WAVE_STEP(0x112, 0xf) ATK_WAVE_STEP(0x114, 0xf) ATK_WAVE_STEP(0x118, 0xf)
+  ATK_WAVE_STEP(0x142, 0xa) ATK_WAVE_STEP(0x143, 0xc)
+#undef ATK_WAVE_STEP
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, kWave - 1);
 }
 __device__ __forceinline__ uint32_t wave_max(uint32_t v) {
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const uint32_t other = (uint32_t)__shfl_xor((int)v, d, kWave);
-    v = other > v ? other : v;
+#define ATK_WAVE_STEP(ctrl, rows)                                                                  \
+  {                                                                                                 \
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, ctrl, rows, 0xf, false);    \
+    v = o > v ? o : v;                                                                              \
   }
-  return v;
+  ATK_WAVE_STEP(0x111, 0xf) ATK_WAVE_STEP(0x112, 0xf) ATK_WAVE_STEP(0x114, 0xf) ATK_WAVE_STEP(0x118, 0xf)
+  ATK_WAVE_STEP(0x142, 0xa) ATK_WAVE_STEP(0x143, 0xc)
+#undef ATK_WAVE_STEP
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, kWave - 1);
 }
 
 struct Found { uint32_t digit, need, count; };  // wave-uniform
@@ -361,17 +369,24 @@ __device__ __forceinline__ Found find_bin_wave(const uint32_t* hist, uint32_t ne
 // largest key differ.)  Whole workgroup of THREADS threads; `red` is
 // 2 * THREADS / 64 words of LDS; contains a barrier, after which every thread
 // holds the result.
+// The ranges this thread looks at, folded: the first half of digit_of_row, for
+// callers that want the loads on their way before they wait for other data.
 template <int THREADS>
-__device__ __forceinline__ void digit_of_row(const uint2* __restrict__ range, uint32_t entries, uint32_t* red,
-                                             uint32_t& low, uint32_t& shift) {
-  constexpr int kWaves = THREADS / kWave;
-  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+__device__ __forceinline__ uint2 fold_ranges(const uint2* __restrict__ range, uint32_t entries) {
   uint32_t lo = ~0u, hi = 0;
-  for (uint32_t g = tid; g < entries; g += THREADS) {
+  for (uint32_t g = threadIdx.x; g < entries; g += THREADS) {
     const uint2 r = range[g];
     lo = r.x < lo ? r.x : lo;
     hi = r.y > hi ? r.y : hi;
   }
+  return make_uint2(lo, hi);
+}
+
+template <int THREADS>
+__device__ __forceinline__ void digit_from_folded(uint2 folded, uint32_t* red, uint32_t& low, uint32_t& shift) {
+  constexpr int kWaves = THREADS / kWave;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  uint32_t lo = folded.x, hi = folded.y;
   lo = wave_min(lo);
   hi = wave_max(hi);
   if (lane == 0) { red[wave] = lo; red[kWaves + wave] = hi; }
@@ -384,6 +399,12 @@ __device__ __forceinline__ void digit_of_row(const uint2* __restrict__ range, ui
   const uint32_t span = lo >= hi ? 0u : 32u - (uint32_t)__builtin_clz(hi - lo);  // bits of the largest offset
   low = lo >= hi ? hi : lo;
   shift = span > (uint32_t)kDigitBits ? span - (uint32_t)kDigitBits : 0u;
+}
+
+template <int THREADS>
+__device__ __forceinline__ void digit_of_row(const uint2* __restrict__ range, uint32_t entries, uint32_t* red,
+                                             uint32_t& low, uint32_t& shift) {
+  digit_from_folded<THREADS>(fold_ranges<THREADS>(range, entries), red, low, shift);
 }
 
 }  // namespace regs

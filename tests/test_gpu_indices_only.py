@@ -26,6 +26,7 @@ CASES = [
     (torch.float32, (8, 1 << 16), 512, 2, 2, True, False),       # streaming kernel, then one workgroup per row
     (torch.float32, (1, 1 << 22), 8192, 4, 2, True, False),      # ... then the chain over many workgroups
     (torch.int16, (1, 1 << 22), 8192, 4, 2, True, False),        # ... with thousands of equal keys at the cut
+    (torch.float32, (1, 1 << 22), 65536, 4, 2, True, False),     # ... too many candidates for one launch: the chain of three
     (torch.uint8, (2, 1 << 23), 1 << 19, 2, 2, True, False),     # ... then passes over many workgroups
     (torch.float32, (2048, 2048), 64, 1, 2, False, False),       # contiguous buckets, then many small selects
 ]
@@ -60,7 +61,7 @@ def test_indices_alone_match_the_full_call_in_every_kernel_family():
         layout = _native.INTERLEAVED if interleaved else _native.BALANCED
         seen += _native.describe(x, k * km, j, k, layout) + "\n"
     for family in ("stream_kernel", "stream_merge_kernel", "contig_kernel", "contig_merge_kernel",
-                   "fused_regs_kernel", "fused_row_kernel", "select_kernel", "chain_emit_kernel",
+                   "fused_regs_kernel", "fused_row_kernel", "select_kernel", "chain_solo_kernel", "chain_emit_kernel",
                    "ms_emit_kernel"):
         assert family in seen, (family, seen)
 

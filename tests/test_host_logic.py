@@ -92,7 +92,7 @@ def test_describe_names_the_planned_kernels():
     c3 = describe(1024, 32768, 1, 2048, 4, 4)
     assert c3.startswith("fused_regs_kernel<f16, J=4, V=4, pos16, PACKED=1> grid=1024 block=512")
     c5 = describe(1, 1 << 26, 0, 16384, 4, 2)
-    assert c5.startswith("stream_kernel<f32, J=4") and "stream_merge_kernel" in c5 and "chain_emit_kernel" in c5
+    assert c5.startswith("stream_kernel<f32, J=4") and "stream_merge_kernel" in c5 and "chain_solo_kernel" in c5
     # a misaligned input: scalar loads, and two kernels instead of the fused one
     odd = describe(1024, 32768, 1, 2048, 4, 4, x=4098)
     assert odd.startswith("stream_kernel<f16, J=4, V=1") and "select_kernel<f16" in odd
