@@ -443,12 +443,8 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
         });
     return;
   }
-  // this thread's candidate of segment g (asked for here and not with the keys:
-  // measured, the index load up there makes the kernel 5 us slower)
-  const uint32_t own = g * kSoloThreads + tid;
+  const uint32_t own = g * kSoloThreads + tid;  // this thread's candidate of segment g
   const bool own_valid = own < k0;
-  const raw_t own_raw = own_valid ? cv[own] : (raw_t)0;
-  const uint32_t own_inv = own_valid ? ~(uint32_t)ci[own] : 0u;
   // survivors above the cut digit (or in it, when it belongs whole) in the
   // segments before this one, and the members of a cut digit listed
   uint32_t before = 0;
@@ -472,6 +468,11 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     ats[n + tid] = ~0u;
   }
   __syncthreads();
+  // This thread's own candidate, asked for together with the listed members'
+  // indices: one trip to memory for both.  (Asked for with the keys at the top,
+  // the index load made the kernel 5 us slower, measured.)
+  const raw_t own_raw = own_valid ? cv[own] : (raw_t)0;
+  const uint32_t own_inv = own_valid ? ~(uint32_t)ci[own] : 0u;
   uint64_t cut = 0;  // the weakest surviving member of B (0: all of them survive)
   if (n != 0) {
     for (uint32_t i = tid; i < n; i += kSoloThreads) words[i] |= (uint64_t)(~(uint32_t)ci[ats[i]]);
