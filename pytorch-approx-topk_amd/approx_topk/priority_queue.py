@@ -129,3 +129,24 @@ def _(
 
 
 topk = torch.ops.approx_topk.topk.default
+
+
+# The reference's ``topk`` is a ``CustomOpDef`` (approx_topk/priority_queue.py:14), whose
+# ``register_fake`` (used at :91) and ``register_autograd`` methods callers may reach for; the
+# overload object carries the same two names, forwarding to ``torch.library``.
+def _register_fake(fn):
+    """Replaces the operator's fake (meta) implementation; usable as a decorator."""
+    torch.library.register_fake("approx_topk::topk", fn, lib=_LIBRARY, allow_override=True)
+    return fn
+
+
+def _register_autograd(backward, /, *, setup_context=None):
+    """Attaches an autograd formula to the operator (``torch.library.register_autograd``).  Once
+    registered, every call goes through autograd's dispatch (about 3 us more per call), which is
+    why none is registered by default: ``approx_topk.experimental.differentiable.topk`` is the
+    opt-in wrapper with the scatter gradient."""
+    torch.library.register_autograd("approx_topk::topk", backward, setup_context=setup_context, lib=_LIBRARY)
+
+
+topk.register_fake = _register_fake
+topk.register_autograd = _register_autograd

@@ -173,3 +173,42 @@ def test_rows_view():
     t, rows, n, step = _native.rows_view(x.movedim(1, -1))
     assert t.is_contiguous() and (rows, n, step) == (30, 4, 4)
 
+
+
+def test_operator_object_offers_register_fake_and_register_autograd():
+    # the reference's `topk` is a CustomOpDef with these two methods (priority_queue.py:14,91); in a child
+    # process, because both registrations change the operator for everything that runs after them
+    import subprocess
+    import sys
+    import textwrap
+
+    code = textwrap.dedent("""
+        import sys
+        sys.path.insert(0, %r)
+        import torch
+        from torch._subclasses.fake_tensor import FakeTensorMode
+        from approx_topk import topk
+
+        @topk.register_fake
+        def _(xs, k, dim, j=None, k_mult=1, interleaved=True, multithread_buckets=False):
+            shape = list(xs.shape)
+            shape[dim] = k
+            return xs.new_empty(shape), xs.new_empty(shape, dtype=torch.int64)
+
+        with FakeTensorMode():
+            v, i = topk(torch.empty(3, 64), 8, -1, 2, 1)
+        assert tuple(v.shape) == (3, 8) and i.dtype == torch.int64
+
+        def setup(ctx, inputs, output):
+            ctx.save_for_backward(output[1])
+            ctx.shape = inputs[0].shape
+
+        def backward(ctx, grad_values, grad_indices):
+            (indices,) = ctx.saved_tensors
+            return torch.zeros(ctx.shape).scatter(-1, indices, grad_values), None, None, None, None, None, None
+
+        topk.register_autograd(backward, setup_context=setup)
+        print("registered")
+    """) % os.path.join(ROOT, "pytorch-approx-topk_amd")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "registered" in out.stdout, out.stderr[-2000:]
