@@ -569,7 +569,10 @@ template <typename E, int J, int V> struct ByteQueue {
 // as +0.0 first (x + 0.0f), as the order has them equal; entries with a zero
 // element are re-read from the row at the end to learn their sign
 // (`fix_zeros`).  Loads are screened for NaN as in the general form.  The empty
-// entry is the double -inf, below every word.
+// entry is the double -inf, below every word.  Words under a zero or a tiny
+// element are subnormal doubles: the kernels run with double-precision
+// subnormals kept (the compiler's default for this target, whatever the fp32
+// mode), and v_max_f64 / v_min_f64 hand back one of their operands unchanged.
 __device__ __forceinline__ double max_f64(double a, double b) {
   double r;
   asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
