@@ -333,6 +333,25 @@ template <uint16_t INF> struct PackedKeyFloat16 {
   __device__ static __forceinline__ bool special(uint32_t screen) {
     return (screen & 0xffffu) > INF || (screen >> 16) > INF;
   }
+  // The same keys in three operations instead of four, with a screen of one
+  // operation instead of two: `screen` accumulates the unsigned max of the raw
+  // halves, which finds the NaNs with the sign bit set (they would key below
+  // -inf and vanish); a NaN without it keys above +inf, stays at the head of its
+  // column's queue whatever else arrives, and is looked for there when the scan
+  // is over (nan_key).  (In the one-kernel path, which is held to 64 registers,
+  // this form was measured slower: it keeps the four-operation one.)
+  __device__ static __forceinline__ uint32_t keys2_lean(uint32_t x, uint32_t& screen) {
+    const uint32_t sign = __builtin_bit_cast(uint32_t, __builtin_bit_cast(atk_short2, x) >> 15);  // 0xFFFF per negative half
+    screen = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(
+                 __builtin_bit_cast(atk_ushort2, screen), __builtin_bit_cast(atk_ushort2, x)));
+    // h ^ 0x8000, or ~h + 1 = -h under the sign: one three-input bit operation, one packed subtract of -1 per negative half
+    const uint32_t flipped = x ^ (sign | 0x80008000u);
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(atk_ushort2, flipped) - __builtin_bit_cast(atk_ushort2, sign));
+  }
+  __device__ static __forceinline__ bool special_lean(uint32_t screen) {
+    return (screen & 0xffffu) > (0x8000u | INF) || (screen >> 16) > (0x8000u | INF);
+  }
+  __device__ static __forceinline__ bool nan_key(uint32_t key) { return key > (0x8000u | INF); }
   // the raw half of a key; a zero key gives +0.0
   __device__ static __forceinline__ uint16_t unkey(uint32_t key) {
     return (uint16_t)((key & 0x8000u) ? (key ^ 0x8000u) : (0u - key));
@@ -349,6 +368,9 @@ template <> struct PackedKey<Elem<ATK_I16>> {
   static constexpr uint32_t kZeroKey = 0x8000u;
   __device__ static __forceinline__ uint32_t keys2(uint32_t x, uint32_t&) { return x ^ 0x80008000u; }
   __device__ static __forceinline__ bool special(uint32_t) { return false; }
+  __device__ static __forceinline__ uint32_t keys2_lean(uint32_t x, uint32_t&) { return x ^ 0x80008000u; }
+  __device__ static __forceinline__ bool special_lean(uint32_t) { return false; }
+  __device__ static __forceinline__ bool nan_key(uint32_t) { return false; }
   __device__ static __forceinline__ uint16_t unkey(uint32_t key) { return (uint16_t)(key ^ 0x8000u); }
   __device__ static __forceinline__ uint32_t exact(uint32_t key) { return key; }
 };
@@ -363,9 +385,18 @@ __device__ __forceinline__ uint32_t med3_u32(uint32_t a, uint32_t b, uint32_t c)
   asm("v_med3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
-template <int J> __device__ __forceinline__ void insert_word(uint32_t (&col)[J], uint32_t word) {
-  ATK_STATIC_FOR(s, J - 1) { col[s] = med3_u32(col[s], word, col[s + 1]); } ATK_STATIC_END;
-  col[J - 1] = col[J - 1] > word ? col[J - 1] : word;
+// FILLED: entries the column is known to hold already (they are its last ones,
+// the others are the empty word 0, below every entry): the slots below them
+// need no work.
+template <int J, int FILLED = J> __device__ __forceinline__ void insert_word(uint32_t (&col)[J], uint32_t word) {
+  ATK_STATIC_FOR(s, J - 1) {
+    if constexpr (s + 1 + FILLED >= J) {
+      if constexpr (s + 1 + FILLED == J) col[s] = col[s + 1] < word ? col[s + 1] : word;  // med3 with an empty col[s]
+      else col[s] = med3_u32(col[s], word, col[s + 1]);
+    }
+  } ATK_STATIC_END;
+  if constexpr (FILLED == 0) col[J - 1] = word;
+  else col[J - 1] = col[J - 1] > word ? col[J - 1] : word;
 }
 
 template <typename E, int J, int V, bool SHIFTED = false> struct PackedQueue {
@@ -407,27 +438,37 @@ template <typename E, int J, int V, bool SHIFTED = false> struct PackedQueue {
   __device__ static __forceinline__ void insert(uint32_t (&col)[J], uint32_t word) { insert_word<J>(col, word); }
   template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
     const uint32_t pinv = low_half(p);
+    // the lean keys and the shorter first inserts: not in the one-kernel path (SHIFTED), see keys2_lean
+    constexpr int F = SHIFTED ? J : FILLED;
     if constexpr (V == 1) {
-      const uint32_t keys = K::keys2(pk.e[0], screen);
-      insert(q[0], (keys << 16) | pinv);
+      const uint32_t keys = SHIFTED ? K::keys2(pk.e[0], screen) : K::keys2_lean(pk.e[0], screen);
+      insert_word<J, F>(q[0], (keys << 16) | pinv);
     } else {
       ATK_STATIC_FOR(d, V / 2) {
         uint32_t x;  // elements 2d (low half) and 2d+1 (high half) as loaded
         __builtin_memcpy(&x, &pk.e[2 * d], 4);
-        const uint32_t keys = K::keys2(x, screen);
-        insert(q[2 * d], (keys << 16) | pinv);
-        insert(q[2 * d + 1], (keys & 0xffff0000u) | pinv);
+        const uint32_t keys = SHIFTED ? K::keys2(x, screen) : K::keys2_lean(x, screen);
+        insert_word<J, F>(q[2 * d], (keys << 16) | pinv);
+        insert_word<J, F>(q[2 * d + 1], (keys & 0xffff0000u) | pinv);
       } ATK_STATIC_END;
     }
   }
   // one more element for column VI, when `valid` (the word 0 changes nothing)
   template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
     uint32_t scr = screen;
-    const uint32_t keys = K::keys2((uint32_t)raw, scr);  // the empty high half screens as +0
+    const uint32_t keys = SHIFTED ? K::keys2((uint32_t)raw, scr) : K::keys2_lean((uint32_t)raw, scr);  // the empty high half screens as +0
     if (valid) screen = scr;
     insert(q[VI], valid ? ((keys << 16) | low_half(p)) : 0u);
   }
-  __device__ __forceinline__ bool poisoned() const { return __ballot(K::special(screen)) != 0; }
+  __device__ __forceinline__ bool poisoned() const {
+    if constexpr (SHIFTED) {
+      return __ballot(K::special(screen)) != 0;
+    } else {
+      bool nan = K::special_lean(screen);
+      ATK_STATIC_FOR(v, V) { nan |= K::nan_key(q[v][J - 1] >> 16); } ATK_STATIC_END;
+      return __ballot(nan) != 0;
+    }
+  }
 
   __device__ __forceinline__ void hand_over(unsigned char* area, uint32_t lane) const {
     uint32_t* h = reinterpret_cast<uint32_t*>(area);
