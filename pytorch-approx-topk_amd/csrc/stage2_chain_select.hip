@@ -350,7 +350,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
 
 
 // ---------------------------------------------------------------------------
-// The chain in one launch, for rows of up to kSoloMaxCandidates candidates.
+// The chain in one launch, for rows of up to kSoloMaxCandidates (32768) candidates.
 //
 // The launches of the chain cost more than their work (4-7 us each against
 // 1-2 us), so for rows short enough every workgroup does the row-wide steps
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
-  __shared__ __align__(16) uint32_t hist[regs::kHistWords];
+  __shared__ __align__(16) uint32_t hist[regs::kBins];  // digit d at word d (find_bin_wave<false>)
   __shared__ select::SharedT<2> sh;
   __shared__ regs::Found found;
   __shared__ uint32_t red[2 * kSoloWaves];
@@ -394,6 +394,9 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   // (the key ranges are asked for first, so that they travel with the keys)
   const uint2 folded = regs::fold_ranges<kSoloThreads>(range + (size_t)row * entries, entries);
   // all keys of the row, NPT per thread (0 past the row's end; `valid` says so)
+  // (The kernel is bound by instruction issue -- sixteen waves on one CU go
+  // through every key of the row -- and short of registers: the keys alone take
+  // up to 64 of its 128.)
   uint32_t key[NPT];
   auto valid = [&](int u) -> bool { return (uint32_t)u * kSoloThreads + tid < k0; };
   {
@@ -403,16 +406,16 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
 #pragma unroll
     for (int u = 0; u < NPT; ++u) key[u] = (uint32_t)E::key(raw[u]);
   }
-  for (uint32_t i = tid; i < (uint32_t)regs::kHistWords; i += kSoloThreads) hist[i] = 0;
+  for (uint32_t i = tid; i < (uint32_t)regs::kBins; i += kSoloThreads) hist[i] = 0;
   if (tid == 0) { list_count = 0; cut_word = 0; }
   uint32_t low, shift;
   regs::digit_from_folded<kSoloThreads>(folded, red, low, shift);  // (its barrier covers the clearing)
 #pragma unroll
   for (int u = 0; u < NPT; ++u)
-    if (valid(u)) atomicAdd(&hist[regs::hist_slot((key[u] - low) >> shift)], 1u);
+    if (valid(u)) atomicAdd(&hist[(key[u] - low) >> shift], 1u);
   __syncthreads();
   if (wave == 0) {
-    const regs::Found f = regs::find_bin_wave(hist, k, k0, lane);
+    const regs::Found f = regs::find_bin_wave<false>(hist, k, k0, lane);
     if (lane == 0) found = f;
   }
   __syncthreads();
@@ -525,7 +528,9 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
 
 // Rows the one-launch form takes: short enough for the keys to sit in registers
 // and for the redundant reads (every workgroup reads the whole row) to stay small.
-constexpr int64_t kSoloMaxCandidates = 64 * kSoloThreads;
+// (With 64 keys per thread the kernel spills: rows of 40000-65536 candidates took
+// 28-30 us against 18 us for the chain of launches.)
+constexpr int64_t kSoloMaxCandidates = 32 * kSoloThreads;
 constexpr int64_t kSoloMaxRedundantBytes = 32ll << 20;
 
 // Rows for which the chain beats one workgroup per row: few rows (one workgroup
@@ -586,8 +591,7 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
                      (uint32_t)k0, (uint32_t)k, pl.groups, index_bits, (const uint2*)range, entries, out, indices)
       if (k0 <= 8 * kSoloThreads) ATK_SOLO(8);
       else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16);
-      else if (k0 <= 32 * kSoloThreads) ATK_SOLO(32);
-      else ATK_SOLO(64);
+      else ATK_SOLO(32);
 #undef ATK_SOLO
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }

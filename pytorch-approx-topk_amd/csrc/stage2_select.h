@@ -331,14 +331,21 @@ struct Found { uint32_t digit, need, count; };  // wave-uniform
 
 // One wave, all 64 lanes: the bin that holds the need-th entry (1-based) of
 // `total` counted from the best digit down, the rank left within it (again from
-// the best) and its population.
+// the best) and its population.  PADDED: the histogram has the layout of
+// hist_slot; else digit d is word d, and the lanes start their 16-byte reads at
+// different quarters of their 128 bytes to stay off each other's banks (two
+// more operations per read and eight address registers for the one reader, for
+// writers that have the registers to spare and many candidates to count).
+template <bool PADDED = true>
 __device__ __forceinline__ Found find_bin_wave(const uint32_t* hist, uint32_t need_from_top, uint32_t total,
                                                uint32_t lane) {
   const uint32_t need = total - need_from_top + 1u;  // counted from the weakest digit up
+  constexpr uint32_t kStride = PADDED ? 36u : 32u;   // words between the chunks of neighbouring lanes
   uint32_t mine = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const uint4 h = *reinterpret_cast<const uint4*>(&hist[lane * 36u + 4u * i]);
+    const uint32_t quarter = PADDED ? (uint32_t)i : ((lane + (uint32_t)i) & 7u);
+    const uint4 h = *reinterpret_cast<const uint4*>(&hist[lane * kStride + 4u * quarter]);
     mine += h.x + h.y + h.z + h.w;
   }
   const uint32_t incl = wave_scan(mine);
@@ -346,7 +353,7 @@ __device__ __forceinline__ Found find_bin_wave(const uint32_t* hist, uint32_t ne
   const int chunk = __builtin_amdgcn_readfirstlane((int)__ffsll((unsigned long long)hit) - 1);
   const uint32_t before = (uint32_t)__builtin_amdgcn_readlane((int)(incl - mine), chunk);
   // the 32 bins of that chunk, one per lane
-  const uint32_t bin = lane < 32u ? hist[(uint32_t)chunk * 36u + lane] : 0u;
+  const uint32_t bin = lane < 32u ? hist[(uint32_t)chunk * kStride + lane] : 0u;
   const uint32_t incl2 = wave_scan(bin);
   const uint32_t left = need - before;
   const uint64_t hit2 = __ballot(incl2 - bin < left && left <= incl2);

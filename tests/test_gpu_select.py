@@ -122,7 +122,7 @@ def _chain_case(rows_spec, k0, k, dtype, bound=1 << 21, seed=0):
                                   (49153, 30000), (65536, 777)])
 def test_chain_select_rows_of_every_kind_together(dtype, k0, k):
     # rows that end by prefix, by a ranked list, by a long list and by the whole-row fallback, in one call;
-    # up to 65536 candidates in one launch (8, 16, 32 or 64 keys per thread), beyond that as a chain of launches
+    # up to 32768 candidates in one launch (8, 16 or 32 keys per thread), beyond that as a chain of launches
     kinds = ["spread", "ties", "equal", "steps", "spread"]
     if dtype == torch.uint8:
         kinds = ["ties", "equal", "steps"]
