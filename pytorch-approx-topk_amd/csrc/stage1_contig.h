@@ -114,7 +114,7 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
   T q[J];
   uint32_t pos[J];
   for (uint32_t it = it0; it < it1; ++it) {
-    // the span this round: all the workgroup's buckets, or one chunk of its only bucket
+    // the span of this trip: all the workgroup's buckets, or one chunk of its only bucket
     uint32_t e0, e1;
     if (g.chunks == 1) {
       e0 = start_of(c0);
