@@ -13,6 +13,10 @@ per-call durations in seconds; input bandwidth is dtype_bytes * n * batch / mean
 (benchmarks/plot_bandwidth.py:41-45).
 
     python pytorch-approx-topk_amd/benchmarks/measure_speed.py [--out results.jsonl] [--quick]
+
+`--reference-rows` times instead the shapes of the measurements the reference keeps of itself
+(fp16, batch 256 or 1, an H100 PCIe: notebooks/data/generic2/measure_speed_approx_finer_multi2.jsonl
+and measure_speed_exact_finer.jsonl), for orientation beside those figures.
 """
 from __future__ import annotations
 
@@ -78,11 +82,59 @@ def time_calls(call: Callable[[int], Any], refresh: Callable[[], None], n_outer:
     return [start.elapsed_time(stop) / 1e3 / n_inner for start, stop in events]
 
 
+# (batch, n, k, j, k_mult) of the reference's own recorded rows, fp16, and the method they timed
+REFERENCE_ROWS = (
+    [("approx_topk.topk", 256, 1 << 20, k, j, 1) for k in (65536, 16384) for j in (1, 2, 4)]
+    + [("approx_topk.topk", 256, 65536, 4096, 4, km) for km in (1, 2, 4, 8)]
+    + [("approx_topk.topk", 256, 262144, 64, 1, 8),
+       ("approx_topk.topk", 1, 4194304, 16384, 4, 2),
+       ("approx_topk.topk", 256, 1 << 22, 4, 1, 2),
+       ("bucketed_argmax.topk_torch", 256, 1 << 20, 65536, 1, 1),
+       ("bucketed_argmax.topk_triton", 256, 1 << 20, 65536, 1, 1),
+       ("bucketed_argmax.topk_torch", 256, 1 << 22, 4096, 1, 1),
+       ("bucketed_argmax.topk_triton", 256, 1 << 22, 4096, 1, 1),
+       ("torch.topk", 256, 1 << 20, 65536, 1, 1)])
+
+
+def reference_rows(out_path: str, quick: bool) -> int:
+    device = torch.cuda.get_device_name()
+    with open(out_path, "w") as out:
+        for name, batch, n, k, j, km in REFERENCE_ROWS:
+            # two or three rotating inputs: together larger than the 256 MiB last-level cache
+            n_inner = 3 if batch * n * 2 < (1 << 30) else 2
+            xs = torch.zeros(n_inner, batch, n, device="cuda", dtype=torch.float16)
+            if name == "approx_topk.topk":
+                call = lambda i: approx_topk(xs[i], k=k, dim=1, j=j, k_mult=km)[0]          # noqa: E731
+            elif name == "bucketed_argmax.topk_torch":
+                call = lambda i: bucketed_argmax.topk_torch(xs[i], k=k, dim=1, interleaved=True)[0]   # noqa: E731
+            elif name == "bucketed_argmax.topk_triton":
+                call = lambda i: bucketed_argmax.topk_triton(xs[i], k=k, dim=1, interleaved=True)[0]  # noqa: E731
+            else:
+                call = lambda i: exact_topk(xs[i], k, 1)[0]                                  # noqa: E731
+            for graph in (False, True):
+                durations = time_calls(call, lambda: xs.normal_(), n_outer=8 if quick else 32, n_inner=n_inner,
+                                       graph=graph, n_warmup=4)
+                mean = sum(durations) / len(durations)
+                row = dict(method=name, args=dict(j=j, k_mult=km), batch_size=batch, topk_size=n, k=k,
+                           dtype="float16", hip_graphs=graph, n_inner=n_inner, duration=durations,
+                           input_GBps=2 * n * batch / mean / 1e9, device=device)
+                print(json.dumps(row), file=out, flush=True)
+                print(f"{name} fp16 [{batch}, {n}] k={k} j={j} k_mult={km} graph={graph}: "
+                      f"{mean * 1e6:.1f} us, {row['input_GBps']:.0f} GB/s", flush=True)
+            del xs
+            torch.cuda.empty_cache()
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default="measure_speed.jsonl")
     ap.add_argument("--quick", action="store_true", help="fewer repetitions")
+    ap.add_argument("--reference-rows", action="store_true",
+                    help="the shapes of the reference's own recorded measurements (fp16) instead of the grid")
     args = ap.parse_args()
+    if args.reference_rows:
+        return reference_rows(args.out, args.quick)
 
     methods: list[tuple[str, Callable, dict]] = [("torch.topk", exact_topk, {})]
     for j in (1, 2, 4):

@@ -53,6 +53,22 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
 
   const int64_t tile_cols = (int64_t)stream::kWave * pl.vec;
   pl.tiles = (uint32_t)((b + tile_cols - 1) / tile_cols);
+  // Few buckets: a sub-row of b elements is all a wave loads at a time here
+  // (this kernel does not fold sub-rows side by side as the streaming kernel
+  // does), so with narrow sub-rows most lanes idle and the few that work walk
+  // the whole row.  Measured against the two-kernel path (fp16 and fp32, 8-256
+  // buckets, k_mult = 2): fp16 [256, 2^22] with 8 buckets 10.2 ms against
+  // 0.36 ms, [2048, 8192] with 32 buckets 29 against 14 us, while rows of a few
+  // KiB still gain from the saved launch (5.5 against 7.7 us).  The sub-row a
+  // call needs grows with the row and with the number of rows; batches of up to
+  // 1 MiB in all are taken whatever their sub-rows.
+  {
+    const size_t sub_row_bytes = (size_t)b * es, row_bytes_ = (size_t)n * es;
+    size_t least = 128;
+    if (row_bytes_ > 16 * 1024) least = 256;
+    if (row_bytes_ > 32 * 1024 || rows >= 2048) least = 512;
+    if ((size_t)rows * row_bytes_ > (1u << 20) && sub_row_bytes < least) return pl;
+  }
   // One launch instead of two, and no candidates parked in HBM: measured over
   // 128-4096 rows of 8192-262144 elements with 256-4096 candidates, this kernel
   // is 5-40 % faster than the two-kernel path for the packed 16-bit types
