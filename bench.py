@@ -37,8 +37,7 @@ MEASURED_TRAFFIC_BYTES = {
     "fused_regs_kernel<f16, J=4, V=4, pos16, PACKED=1> grid=1024 block=512 tiles=8 split=1 lds=32768 staged": 123_255_808,
     "fused_regs_kernel<f32, J=1, V=4, pos16, PACKED=0> grid=256 block=512 tiles=2 split=4 lds=19584 staged": 134_724_608,
     "stream_kernel<f32, J=4, V=4, W=4, U=8, RUN=0, PACKED=0> grid=256 block=256 fold=1 slabs=8 + "
-    "stream_merge_kernel<f32, J=4> + [chain_range_kernel<f32> unless stage 1 left key ranges] + "
-    "chain_solo_kernel<f32> grid=32 block=1024": 275_389_132,
+    "stream_merge_kernel<f32, J=4> + chain_solo_kernel<f32> grid=32 block=1024": 275_389_132,
 }
 
 # name -> (rows, n, dtype, k, j, k_mult, seed)

@@ -23,9 +23,14 @@
 //
 // A candidate is the 64-bit word (order key, inverted index): a greater word is a
 // better candidate and no two are equal, so that ties go to the lower index.
-// A row whose digit B holds more candidates than the list takes is selected by
-// its first workgroup alone, with the block-wide radix select over all of its
-// candidates.  When stage 1 ends in kernels that can leave key ranges and the
+// When the digit B holds more candidates than a workgroup's LDS list takes
+// (kListCap; keys that crowd into a small part of their span: heavy tails,
+// outliers), the members of B are counted again by the next 11 bits of their
+// offsets, and so on until the cut digit fits or no bits are left (every emit
+// workgroup does this over the row's list in global memory, which holds all of
+// B).  Only a row with more than kListCap candidates of one and the same key
+// around the cut is selected by its first workgroup alone, with the block-wide
+// radix select over all of its candidates.  When stage 1 ends in kernels that can leave key ranges and the
 // histogram behind (KeyRangeOut: the streaming kernel's slabs and their merge),
 // the range and hist launches are skipped.  Results are those of the
 // one-workgroup kernel: same survivors, same order.
@@ -47,13 +52,12 @@ constexpr uint32_t kRankDirect = 256;                 // lists up to this size a
 
 // Per-row words in the workspace.
 struct RowState {
-  uint32_t list_count;  // candidates appended to the list (may exceed kListCap: then the row is left to the fallback)
+  uint32_t list_count;  // candidates appended to the row's list
   uint32_t digit;       // B
   uint32_t need;        // members of B that belong to the result
   uint32_t count;       // members of B
   uint32_t shift, low;  // the digit is (key - low) >> shift
-  uint32_t fallback;    // != 0: the one-workgroup kernel takes this row
-  uint32_t unused;
+  uint32_t unused[2];
 };
 
 // Shares per row whose key ranges the workspace has room for: the chain's own
@@ -108,7 +112,7 @@ __global__ __launch_bounds__(kThreads) void chain_range_kernel(const typename E:
   // this workgroup's share of the row's histogram, and the row's state
   uint32_t* h = hist + (size_t)row * regs::kHistWords;
   for (uint32_t i = g * kThreads + tid; i < regs::kHistWords; i += groups * kThreads) h[i] = 0;
-  if (g == 0 && tid == 0) state[row] = RowState{0, 0, 0, 0, 0, 0, 0, 0};
+  if (g == 0 && tid == 0) state[row] = RowState{0, 0, 0, 0, 0, 0, {0, 0}};
   __syncthreads();
   if (tid == 0) {
 #pragma unroll
@@ -154,7 +158,8 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
     uint64_t* __restrict__ list_word, uint32_t* __restrict__ list_at) {
   __shared__ __align__(16) uint32_t local[regs::kHistWords];
   __shared__ regs::Found found;
-  __shared__ uint32_t wave_above[kWaves];
+  __shared__ uint32_t wave_above[kWaves], wave_listed[kWaves];
+  __shared__ uint32_t list_base;
   __shared__ uint32_t red[2 * kWaves];
   const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
   const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
@@ -177,32 +182,44 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
   __syncthreads();
   const regs::Found f = found;
   uint32_t mine = 0;
+  bool member[kPerThread];  // of a digit that is cut: ranked later, from the row's list
+  uint32_t listed = 0;
 #pragma unroll
   for (int u = 0; u < kPerThread; ++u) {
-    if (!valid[u]) continue;
     const uint32_t d = (key[u] - low) >> shift;
     // survivors known now: above B, and all of B when none of it is cut
-    mine += (d > f.digit || (d == f.digit && f.need == f.count)) ? 1u : 0u;
-    if (d == f.digit && f.need != f.count) {  // the digit is cut: its members are ranked later
-      const uint32_t slot = atomicAdd(&state[row].list_count, 1u);
-      if (slot < kListCap) {
-        list_word[(size_t)row * kListCap + slot] = ((uint64_t)key[u] << 32) | (uint64_t)inv[u];
-        list_at[(size_t)row * kListCap + slot] = first + u * kThreads;
-      }
-    }
+    mine += (valid[u] && (d > f.digit || (d == f.digit && f.need == f.count))) ? 1u : 0u;
+    member[u] = valid[u] && d == f.digit && f.need != f.count;
+    listed += member[u] ? 1u : 0u;
   }
   const uint32_t incl = regs::wave_scan(mine);
-  if (lane == select::kWave - 1) wave_above[wave] = incl;
+  const uint32_t listed_incl = regs::wave_scan(listed);
+  if (lane == select::kWave - 1) { wave_above[wave] = incl; wave_listed[wave] = listed_incl; }
   __syncthreads();
   if (tid == 0) {
-    uint32_t total = 0;
+    uint32_t total = 0, total_listed = 0;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) total += wave_above[w];
+    for (int w = 0; w < kWaves; ++w) { total += wave_above[w]; total_listed += wave_listed[w]; }
     above[(size_t)row * groups + g] = total;
+    // one reservation in the row's list for the whole workgroup (the row's list takes
+    // all k0 candidates, so every member has a place)
+    list_base = total_listed != 0 ? atomicAdd(&state[row].list_count, total_listed) : 0u;
     if (g == 0) {
       RowState* s = &state[row];
       s->digit = f.digit; s->need = f.need; s->count = f.count; s->shift = shift; s->low = low;
-      s->fallback = (f.need != f.count && f.count > kListCap) ? 1u : 0u;
+    }
+  }
+  if (f.need == f.count) return;  // (uniform) nothing is listed
+  __syncthreads();
+  uint32_t slot = list_base + listed_incl - listed;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) slot += (uint32_t)w < wave ? wave_listed[w] : 0u;
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    if (member[u]) {
+      list_word[(size_t)row * k0 + slot] = ((uint64_t)key[u] << 32) | (uint64_t)inv[u];
+      list_at[(size_t)row * k0 + slot] = first + u * kThreads;
+      ++slot;
     }
   }
 }
@@ -220,20 +237,53 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
   __shared__ uint64_t cut_word;
   __shared__ uint32_t listed_before;
   __shared__ uint32_t wave_kept[kPerThread][kWaves];
+  __shared__ regs::Found found;
+  __shared__ uint32_t lds_count;
   const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
   const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
+  const uint64_t* lw = list_word + (size_t)row * k0;
+  const uint32_t* la = list_at + (size_t)row * k0;
   // asked for before the row's state is known: the start of the list (most lists end within it) and
   // the survivors counted for the segments before this one
-  const uint64_t early_word = list_word[(size_t)row * kListCap + tid];
-  const uint32_t early_at = list_at[(size_t)row * kListCap + tid];
+  const uint64_t early_word = lw[tid];
+  const uint32_t early_at = la[tid];
   uint32_t counted = 0;
   for (uint32_t p = tid; p < g; p += kThreads) counted += above[(size_t)row * groups + p];
   const RowState s = state[row];
-  if (s.fallback != 0) {
-    // The cut digit holds more candidates than the list: the row's first
+  uint32_t digit = s.digit, shift = s.shift, need = s.need, count = s.count;
+  const uint32_t listed = need != count ? count : 0u;  // entries of the row's list: all members of B
+  if (listed > kListCap) {
+    // More members than a workgroup ranks: they are counted again by the next bits of their
+    // offsets, which narrows the digit that is cut, until its members fit (the histogram borrows
+    // the memory of the LDS list, which is filled afterwards).
+    uint32_t* local = reinterpret_cast<uint32_t*>(dyn_lds);
+    while (need != count && count > kListCap && shift != 0) {
+      const uint32_t finer = shift > (uint32_t)regs::kDigitBits ? shift - (uint32_t)regs::kDigitBits : 0u;
+      const uint32_t mask = (1u << (shift - finer)) - 1u;
+      for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = 0;
+      __syncthreads();
+      for (uint32_t i = tid; i < listed; i += kThreads) {
+        const uint32_t off = (uint32_t)(lw[i] >> 32) - s.low;
+        if ((off >> shift) == digit) atomicAdd(&local[regs::hist_slot((off >> finer) & mask)], 1u);
+      }
+      __syncthreads();
+      if (wave == 0) {
+        const regs::Found f = regs::find_bin_wave(local, need, count, lane);
+        if (lane == 0) found = f;
+      }
+      __syncthreads();
+      const regs::Found f = found;
+      digit = (digit << (shift - finer)) | f.digit;
+      shift = finer;
+      need = f.need;
+      count = f.count;
+    }
+  }
+  if (need != count && count > kListCap) {
+    // More than kListCap candidates of one key around the cut: the row's first
     // workgroup runs the block-wide radix select of stage2_select.h over all of
-    // the row's candidates, read from global memory (slow, but only rows with
-    // thousands of equal keys around the cut come here).
+    // the row's candidates, read from global memory (slow, for rows with
+    // thousands of equal keys only).
     if (g != 0) return;
     const raw_t* rv = cand_values + (int64_t)row * k0;
     const int64_t* ri = cand_indices + (int64_t)row * k0;
@@ -256,8 +306,8 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
         });
     return;
   }
-  const bool cut_digit = s.need != s.count;  // else every member of B survives
-  const uint32_t n = cut_digit ? s.count : 0u;
+  const bool cut_digit = need != count;  // else every member of the digit survives
+  const uint32_t n = cut_digit ? count : 0u;  // members ranked here, in LDS
   uint64_t* words = reinterpret_cast<uint64_t*>(dyn_lds);
   uint32_t* ats = reinterpret_cast<uint32_t*>(dyn_lds + (size_t)kListCap * sizeof(uint64_t));
   const uint32_t first = g * kSegment + tid;
@@ -274,11 +324,33 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
     inv[u] = valid[u] ? ~(uint32_t)ci[first + u * kThreads] : 0u;
   }
   // entries past the list's end count as beating nothing (ranking reads the list in groups of eight)
-  words[tid] = tid < n ? early_word : 0ull;
-  ats[tid] = tid < n ? early_at : ~0u;
-  for (uint32_t i = tid + kThreads; i < ((n + 7u) & ~7u); i += kThreads) {
-    words[i] = i < n ? list_word[(size_t)row * kListCap + i] : 0ull;
-    ats[i] = i < n ? list_at[(size_t)row * kListCap + i] : ~0u;
+  if (listed <= kListCap) {
+    words[tid] = tid < n ? early_word : 0ull;
+    ats[tid] = tid < n ? early_at : ~0u;
+    for (uint32_t i = tid + kThreads; i < ((n + 7u) & ~7u); i += kThreads) {
+      words[i] = i < n ? lw[i] : 0ull;
+      ats[i] = i < n ? la[i] : ~0u;
+    }
+  } else {
+    // of the row's list, the members of the narrowed digit are ranked; those above it survive
+    if (tid == 0) lds_count = 0;
+    __syncthreads();  // (also: the histogram in this memory has been read)
+    for (uint32_t i = tid; i < listed; i += kThreads) {
+      const uint64_t w = lw[i];
+      const uint32_t at = la[i];
+      const uint32_t d = ((uint32_t)(w >> 32) - s.low) >> shift;
+      if (d > digit || (d == digit && !cut_digit)) {
+        counted += at < g * kSegment ? 1u : 0u;
+      } else if (d == digit) {
+        const uint32_t slot = atomicAdd(&lds_count, 1u);
+        words[slot] = w;
+        ats[slot] = at;
+      }
+    }
+    if (tid < 8u && n + tid < ((n + 7u) & ~7u)) {
+      words[n + tid] = 0ull;
+      ats[n + tid] = ~0u;
+    }
   }
   if (tid == 0) { cut_word = 0; listed_before = 0; }
   __syncthreads();
@@ -296,7 +368,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
 #pragma unroll
           for (int e = 0; e < 8; ++e) better += got[e] > mine ? 1u : 0u;
         }
-        if (better + 1 == s.need) cut_word = mine;
+        if (better + 1 == need) cut_word = mine;
       }
       __syncthreads();
       cut = cut_word;
@@ -304,7 +376,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
       // a longer list: the block-wide radix select over its words (all distinct)
       auto key_at = [&](uint32_t i) -> uint64_t { return words[i]; };
       auto index_at = [&](uint32_t) -> uint64_t { return 0; };
-      cut = select::find_cut<uint64_t, 64>(sh, n, s.need, 1, key_at, index_at).T;
+      cut = select::find_cut<uint64_t, 64>(sh, n, need, 1, key_at, index_at).T;
     }
     // listed survivors of the segments before this one
     uint32_t before = 0;
@@ -317,8 +389,8 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
 #pragma unroll
   for (int u = 0; u < kPerThread; ++u) {
     const uint32_t key = (uint32_t)E::key(raw[u]);
-    const uint32_t d = (key - s.low) >> s.shift;
-    sel[u] = valid[u] && (d > s.digit || (d == s.digit && (((uint64_t)key << 32) | inv[u]) >= cut));
+    const uint32_t d = (key - s.low) >> shift;
+    sel[u] = valid[u] && (d > digit || (d == digit && (((uint64_t)key << 32) | inv[u]) >= cut));
     const uint64_t m = __ballot(sel[u]);
     if (lane == 0) wave_kept[u][wave] = (uint32_t)__popcll(m);
   }
@@ -361,15 +433,15 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
 // best, lists the members of B in LDS and ranks them, counts the survivors of
 // the segments before its own from the keys it holds, and writes its segment.
 // The row's keys are read groups-times over (32 x 128 KiB at fp32 [1, 32768]),
-// from L2 for the most part.  The key ranges come from stage 1 or from a
-// chain_range_kernel launch, as before.
+// from L2 for the most part.  The key ranges come from stage 1, or from the
+// keys themselves when stage 1 left none.
 // ---------------------------------------------------------------------------
 constexpr int kSoloThreads = 1024;  // == kSegment
 constexpr int kSoloWaves = kSoloThreads / select::kWave;
 constexpr uint32_t kSoloRankDirect = 512;
 static_assert((uint32_t)kSoloThreads == kSegment, "a thread's u-th candidate lies in segment u");
 
-template <typename E, int NPT>
+template <typename E, int NPT, bool OWN_RANGE>
 __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t groups, int index_bits, const uint2* __restrict__ range, uint32_t entries,
@@ -391,8 +463,10 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   const raw_t* cv = cand_values + (int64_t)row * k0;
   const int64_t* ci = cand_indices + (int64_t)row * k0;
 
-  // (the key ranges are asked for first, so that they travel with the keys)
-  const uint2 folded = regs::fold_ranges<kSoloThreads>(range + (size_t)row * entries, entries);
+  // (the key ranges are asked for first, so that they travel with the keys; OWN_RANGE:
+  // stage 1 left none, and the range is that of the keys read below)
+  uint2 folded = make_uint2(~0u, 0u);
+  if constexpr (!OWN_RANGE) folded = regs::fold_ranges<kSoloThreads>(range + (size_t)row * entries, entries);
   // all keys of the row, NPT per thread (0 past the row's end; `valid` says so)
   // (The kernel is bound by instruction issue -- sixteen waves on one CU go
   // through every key of the row -- and short of registers: the keys alone take
@@ -408,6 +482,15 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   }
   for (uint32_t i = tid; i < (uint32_t)regs::kBins; i += kSoloThreads) hist[i] = 0;
   if (tid == 0) { list_count = 0; cut_word = 0; }
+  if constexpr (OWN_RANGE) {
+#pragma unroll
+    for (int u = 0; u < NPT; ++u) {
+      if (valid(u)) {
+        folded.x = key[u] < folded.x ? key[u] : folded.x;
+        folded.y = key[u] > folded.y ? key[u] : folded.y;
+      }
+    }
+  }
   uint32_t low, shift;
   regs::digit_from_folded<kSoloThreads>(folded, red, low, shift);  // (its barrier covers the clearing)
 #pragma unroll
@@ -419,13 +502,39 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     if (lane == 0) found = f;
   }
   __syncthreads();
-  const regs::Found f = found;
+  regs::Found f = found;
+  // The cut digit holds more candidates than the list: they are counted again by
+  // the next bits of their offsets, which narrows the digit, until its members
+  // fit or no bits are left.
+  while (f.need != f.count && f.count > kListCap && shift != 0) {
+    const uint32_t finer = shift > (uint32_t)regs::kDigitBits ? shift - (uint32_t)regs::kDigitBits : 0u;
+    const uint32_t mask = (1u << (shift - finer)) - 1u;
+    __syncthreads();  // everyone has read `found`, wave 0 the histogram
+    for (uint32_t i = tid; i < (uint32_t)regs::kBins; i += kSoloThreads) hist[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NPT; ++u) {
+      const uint32_t off = key[u] - low;
+      if (valid(u) && (off >> shift) == f.digit) atomicAdd(&hist[(off >> finer) & mask], 1u);
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const regs::Found f2 = regs::find_bin_wave<false>(hist, f.need, f.count, lane);
+      if (lane == 0) found = f2;
+    }
+    __syncthreads();
+    const regs::Found f2 = found;
+    f.digit = (f.digit << (shift - finer)) | f2.digit;
+    f.need = f2.need;
+    f.count = f2.count;
+    shift = finer;
+  }
   const bool cut_digit = f.need != f.count;  // else every member of B survives
   if (cut_digit && f.count > kListCap) {
-    // The cut digit holds more candidates than the list: the row's first
+    // More than kListCap candidates of one key around the cut: the row's first
     // workgroup runs the block-wide radix select of stage2_select.h over all of
-    // the row's candidates, read from global memory (slow, but only rows with
-    // thousands of equal keys around the cut come here).
+    // the row's candidates, read from global memory (slow, for rows with
+    // thousands of equal keys only).
     if (g != 0) return;
     auto key_at = [&](uint32_t i) -> key_t { return E::key(cv[i]); };
     auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)ci[i]; };
@@ -526,36 +635,48 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   }
 }
 
-// Rows the one-launch form takes: short enough for the keys to sit in registers
-// and for the redundant reads (every workgroup reads the whole row) to stay small.
+// Rows the one-launch form takes: short enough for the keys to sit in registers,
+// and few enough that all workgroups run at once, one per CU (a second round
+// doubles the time: 16 rows of 32768 fp16 candidates took 32.6 us in 512
+// workgroups, 8 rows 18.4 us in 256).
 // (With 64 keys per thread the kernel spills: rows of 40000-65536 candidates took
 // 28-30 us against 18 us for the chain of launches.)
 constexpr int64_t kSoloMaxCandidates = 32 * kSoloThreads;
-constexpr int64_t kSoloMaxRedundantBytes = 32ll << 20;
+constexpr int64_t kSoloMaxWorkgroups = 256;
 
 // Rows for which the chain beats one workgroup per row: few rows (one workgroup
 // per row already fills the GPU with many), enough candidates that a single CU
-// is what bounds them, keys of at most 32 bits and indices below 2^31.
-constexpr int64_t kChainMinCandidates = 8192;
+// is what bounds them, keys of at most 32 bits and indices below 2^31.  Measured,
+// select alone, microseconds, fp16 / fp32, chain against one workgroup per row:
+// 16 rows of 16384: 14.6 / 18.9 against 16.3 / 18.3; 32 rows of 16384: 21.7 / 35.2;
+// 16 rows of 65536: 34 / 33 against 70 / 73; 32 rows of 65536: 52 / 49;
+// 64 rows of 65536: 92 / 89; 32 rows of 131072: 119 / 125 against 121 / 125.
+constexpr int64_t kChainMinCandidates = 10240;  // (8192: 11.8 us against 10.5 for one workgroup)
 constexpr int64_t kChainMaxCandidates = 1 << 17;
-constexpr int64_t kChainMaxRows = 64;
+constexpr int64_t kChainMaxRows = 16;
+constexpr int64_t kChainMaxRowsLong = 32;  // rows of kChainLong candidates and more
+constexpr int64_t kChainLong = 1 << 16;
 
 ChainPlan plan_chain(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype) {
   ChainPlan pl{};
   pl.use = false;
   const int es = elem_bytes(dtype);
-  if (es == 0 || es > 4 || rows <= 0 || rows > kChainMaxRows || k <= 0 || k >= k0) return pl;
+  if (es == 0 || es > 4 || rows <= 0 || k <= 0 || k >= k0) return pl;
+  if (rows > (k0 >= kChainLong ? kChainMaxRowsLong : kChainMaxRows)) return pl;
   if (k0 < kChainMinCandidates || k0 > kChainMaxCandidates || index_bound > 0x7fffffffll) return pl;
   pl.groups = (uint32_t)((k0 + kSegment - 1) / kSegment);
-  pl.solo = k0 <= kSoloMaxCandidates && rows * (int64_t)pl.groups * k0 * es <= kSoloMaxRedundantBytes;
+  pl.solo = k0 <= kSoloMaxCandidates && rows * (int64_t)pl.groups <= kSoloMaxWorkgroups;
   pl.range_off = 0;
   pl.range_capacity = pl.groups > kRangeCapacity ? pl.groups : kRangeCapacity;
   pl.hist_off = align_up((size_t)rows * pl.range_capacity * sizeof(uint2), 256);
   pl.state_off = pl.hist_off + align_up((size_t)rows * regs::kHistWords * sizeof(uint32_t), 256);
   pl.above_off = pl.state_off + align_up((size_t)rows * sizeof(RowState), 256);
   pl.list_word_off = pl.above_off + align_up((size_t)rows * pl.groups * sizeof(uint32_t), 256);
-  pl.list_at_off = pl.list_word_off + align_up((size_t)rows * kListCap * sizeof(uint64_t), 256);
-  pl.total = pl.list_at_off + align_up((size_t)rows * kListCap * sizeof(uint32_t), 256);
+  // the row's list takes every candidate of the row (all may share the cut digit); the
+  // one-launch form keeps its list in LDS
+  const size_t listed = pl.solo ? 0 : (size_t)rows * (size_t)k0;
+  pl.list_at_off = pl.list_word_off + align_up(listed * sizeof(uint64_t), 256);
+  pl.total = pl.list_at_off + align_up(listed * sizeof(uint32_t), 256);
   pl.use = true;
   return pl;
 }
@@ -577,7 +698,7 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
     const dim3 grid((unsigned)(rows * pl.groups)), block(kThreads);
     const size_t emit_lds = (size_t)kListCap * (sizeof(uint64_t) + sizeof(uint32_t));
     uint32_t entries = range_entries;
-    if (entries == 0) {  // stage 1 left no key ranges
+    if (entries == 0 && !pl.solo) {  // stage 1 left no key ranges
       hipLaunchKernelGGL((chain_range_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups, range, hist,
                          state);
       entries = pl.groups;
@@ -586,12 +707,18 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
       const size_t solo_lds = (size_t)(kListCap + 8) * (sizeof(uint64_t) + sizeof(uint32_t));
       const dim3 solo_block(kSoloThreads);
       raw_t* out = static_cast<raw_t*>(values);
-#define ATK_SOLO(NPT)                                                                                            \
-  hipLaunchKernelGGL((chain_solo_kernel<E, NPT>), grid, solo_block, solo_lds, stream, cv, cand_indices,          \
+#define ATK_SOLO(NPT, OWN)                                                                                       \
+  hipLaunchKernelGGL((chain_solo_kernel<E, NPT, OWN>), grid, solo_block, solo_lds, stream, cv, cand_indices,     \
                      (uint32_t)k0, (uint32_t)k, pl.groups, index_bits, (const uint2*)range, entries, out, indices)
-      if (k0 <= 8 * kSoloThreads) ATK_SOLO(8);
-      else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16);
-      else ATK_SOLO(32);
+      if (entries != 0) {
+        if (k0 <= 8 * kSoloThreads) ATK_SOLO(8, false);
+        else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16, false);
+        else ATK_SOLO(32, false);
+      } else {
+        if (k0 <= 8 * kSoloThreads) ATK_SOLO(8, true);
+        else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16, true);
+        else ATK_SOLO(32, true);
+      }
 #undef ATK_SOLO
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }
@@ -624,7 +751,7 @@ bool describe_chain_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bo
   if (!pl.use) return false;
   const std::string t = dtype_name(dtype);
   if (pl.solo) {
-    out += "[chain_range_kernel<" + t + "> unless stage 1 left key ranges] + chain_solo_kernel<" + t + "> grid=" +
+    out += "chain_solo_kernel<" + t + "> grid=" +
            std::to_string(rows * (int64_t)pl.groups) + " block=" + std::to_string(kSoloThreads);
     return true;
   }

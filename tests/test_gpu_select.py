@@ -107,6 +107,20 @@ def _chain_case(rows_spec, k0, k, dtype, bound=1 << 21, seed=0):
             r = torch.randint(-3, 4, (k0,), generator=g)
         elif kind == "equal":
             r = torch.full((k0,), 2.0)
+        elif kind in ("outliers", "tied outliers", "crowded"):
+            # two values far from all others stretch the span of the keys: nearly every candidate
+            # shares the leading digit of its offset, and the cut is found some digits further down
+            if kind == "tied outliers":
+                r = torch.randint(-3, 4, (k0,), generator=g).double()
+            elif kind == "crowded" and dtype.is_floating_point:
+                r = 1.0 + torch.randn(k0, generator=g).double() * 1e-4
+            elif dtype.is_floating_point:
+                r = torch.randn(k0, generator=g).double()
+            else:
+                r = torch.randint(-30000, 30000, (k0,), generator=g).double()
+            big = float(torch.finfo(dtype).max) / 2 if dtype.is_floating_point else float(torch.iinfo(dtype).max)
+            at = torch.randperm(k0, generator=g)[:2]
+            r[at[0]], r[at[1]] = big, -big
         else:
             r = (torch.arange(k0) // 3000).float()[torch.randperm(k0, generator=g)]
         rows.append(r.to(dtype))
@@ -127,6 +141,15 @@ def test_chain_select_rows_of_every_kind_together(dtype, k0, k):
     if dtype == torch.uint8:
         kinds = ["ties", "equal", "steps"]
     _chain_case(kinds, k0, k, dtype, seed=k0 + k)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.int32])
+@pytest.mark.parametrize("k0,k", [(8192, 4000), (16384, 100), (32768, 16384), (20000, 19000), (65536, 8192),
+                                  (131072, 60000), (49153, 3)])
+def test_chain_select_narrows_a_crowded_digit(dtype, k0, k):
+    # the digit that is cut holds far more candidates than a workgroup ranks: it is narrowed by the
+    # next bits, several times over, down to single keys (then the whole-row path takes the row)
+    _chain_case(["outliers", "crowded", "tied outliers", "spread"], k0, k, dtype, seed=k0 * 3 + k)
 
 
 def test_chain_select_needs_no_cut_when_the_digit_belongs_whole():
