@@ -60,14 +60,18 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   // buckets, k_mult = 2): fp16 [256, 2^22] with 8 buckets 10.2 ms against
   // 0.36 ms, [2048, 8192] with 32 buckets 29 against 14 us, while rows of a few
   // KiB still gain from the saved launch (5.5 against 7.7 us).  The sub-row a
-  // call needs grows with the row and with the number of rows; batches of up to
-  // 1 MiB in all are taken whatever their sub-rows.
+  // call needs grows with the row and with the number of rows.  Batches of up to
+  // 1 MiB in all are bound by launches, not by bytes: there this kernel takes
+  // 5 us + 11 ns per sub-row of the row ([4, 32768] with 4 buckets: 94-118 us)
+  // against 8-15 us for the two kernels whatever the shape, and narrow sub-rows
+  // are taken while the row has fewer than 256 of them.
   {
     const size_t sub_row_bytes = (size_t)b * es, row_bytes_ = (size_t)n * es;
     size_t least = 128;
     if (row_bytes_ > 16 * 1024) least = 256;
     if (row_bytes_ > 32 * 1024 || rows >= 2048) least = 512;
-    if ((size_t)rows * row_bytes_ > (1u << 20) && sub_row_bytes < least) return pl;
+    const bool small_batch = (size_t)rows * row_bytes_ <= (1u << 20);
+    if (sub_row_bytes < least && (!small_batch || full >= 256)) return pl;
   }
   // One launch instead of two, and no candidates parked in HBM: measured over
   // 128-4096 rows of 8192-262144 elements with 256-4096 candidates, this kernel

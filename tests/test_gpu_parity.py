@@ -372,6 +372,19 @@ def test_few_long_buckets_all_dtypes_with_ties(dtype, j, k_mult, n):
     _check(x, 12, -1, j=j, k_mult=k_mult)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("rows,n,k,j,k_mult", [
+    (4, 32768, 4, 2, 2), (16, 32768, 4, 4, 8), (2, 4096, 2, 1, 2), (64, 1024, 4, 1, 2), (64, 1 << 18, 4, 1, 2),
+    (300, 8192, 16, 1, 2), (2100, 2048, 16, 2, 4),
+])
+def test_few_buckets_with_a_second_stage(dtype, rows, n, k, j, k_mult):
+    # aligned rows whose candidates would fit the one-kernel path: narrow sub-rows go to the folding
+    # streaming kernel instead, short rows of few sub-rows stay
+    g = torch.Generator().manual_seed(rows + n + k)
+    x = (torch.randint(-50, 50, (rows, n), generator=g) / 8).to(dtype)
+    _check(x, k, -1, j=j, k_mult=k_mult)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
 @pytest.mark.parametrize("n", [40000, 4100])
 def test_few_long_buckets_special_values(dtype, n):

@@ -93,6 +93,16 @@ def test_describe_names_the_planned_kernels():
     assert c3.startswith("fused_regs_kernel<f16, J=4, V=4, pos16, PACKED=1> grid=1024 block=512")
     c5 = describe(1, 1 << 26, 0, 16384, 4, 2)
     assert c5.startswith("stream_kernel<f32, J=4") and "stream_merge_kernel" in c5 and "chain_solo_kernel" in c5
+    # few buckets (narrow sub-rows): the streaming kernel, which folds sub-rows side by side,
+    # not the one-kernel path, whose lanes would idle; short rows of few sub-rows stay with it
+    assert describe(256, 1 << 22, 1, 4, 1, 2).startswith("stream_kernel<f16, J=1")
+    assert describe(4, 32768, 1, 4, 2, 2).startswith("stream_kernel<f16, J=2")
+    assert describe(4, 32768, 0, 4, 4, 8).startswith("stream_kernel<f32, J=4")
+    assert describe(64, 1024, 1, 8, 1, 2).startswith("fused_regs_kernel<f16, J=1")
+    # the select over several workgroups per row: few rows only, one launch up to 32768 candidates
+    assert "chain_solo_kernel<f32> grid=16 " in describe(1, 1 << 24, 0, 8192, 2, 2)
+    assert "chain_emit_kernel<f32> grid=512 " in describe(8, 1 << 22, 0, 32768, 2, 2)
+    assert "chain_" not in describe(64, 1 << 18, 0, 16384, 2, 8)
     # a misaligned input: scalar loads, and two kernels instead of the fused one
     odd = describe(1024, 32768, 1, 2048, 4, 4, x=4098)
     assert odd.startswith("stream_kernel<f16, J=4, V=1") and "select_kernel<f16" in odd
