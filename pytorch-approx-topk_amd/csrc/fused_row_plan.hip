@@ -15,6 +15,14 @@ constexpr size_t kSoloRow = 256 * 1024;
 // Dynamic LDS a workgroup may use (candidates + hand-over); the select's own
 // block adds about 9 KiB.
 constexpr size_t kLdsBudget = 64 * 1024;
+// For rows of up to 256 KiB the candidates may take twice that (one workgroup
+// per CU then): the alternative parks them in HBM and selects with one
+// workgroup per row as well.  Measured with the larger budget: fp16 [256, 65536]
+// k0=32768 71 -> 52 us, [1024, 65536] 312 -> 196 us, fp32 [256, 65536] k0=16384
+// 52 -> 39 us; longer rows lose (fp16 [128, 2^20] k0=32768 87 -> 115 us, fp32
+// [1024, 131072] k0=16384 195 -> 208 us).
+constexpr size_t kLdsBudgetShortRows = 128 * 1024;
+constexpr size_t kShortRowsForLds = 256 * 1024;
 // Most waves per workgroup.  Measured over shapes from [4096, 4096] to
 // [256, 65536]: 8 beats 16 (more workgroups per CU, in different phases, and
 // cheaper barriers) and is never far behind 4.
@@ -90,7 +98,8 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   const int skey = (dtype == ATK_U8 || dtype == ATK_I8) ? 2 : es;  // stored key width
   const size_t cand_bytes = (((size_t)k0 * skey + 15) & ~(size_t)15) +
                             (((size_t)k0 * (pl.pos16 ? 2 : 4) + 15) & ~(size_t)15);
-  if (cand_bytes > kLdsBudget) return pl;
+  const size_t lds_budget = row_bytes <= kShortRowsForLds ? kLdsBudgetShortRows : kLdsBudget;
+  if (cand_bytes > lds_budget) return pl;
 
   // Waves sharing a tile: as many as keep each share at least max(j, 8)
   // sub-rows long, the workgroup within its wave limit and LDS within budget.
@@ -110,7 +119,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   uint32_t split = 1;
   if (pl.tiles < kMaxWaves) {
     for (uint32_t cand = 2; cand * pl.tiles <= kMaxWaves; cand *= 2) {
-      if (full / cand < min_run || lds_need(cand) > kLdsBudget) break;
+      if (full / cand < min_run || lds_need(cand) > lds_budget) break;
       split = cand;
     }
   }

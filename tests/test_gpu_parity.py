@@ -280,6 +280,20 @@ def test_fused_rows_shapes(n, k, j, k_mult):
     _check(cpu_randn((136, n), n + k), k, -1, j=j, k_mult=k_mult)
 
 
+@pytest.mark.parametrize("dtype,rows,n,k,j,k_mult", [
+    (torch.float16, 130, 65536, 4096, 4, 8),     # 32768 candidates: 128 KiB of LDS
+    (torch.bfloat16, 9, 65536, 3072, 1, 8),      # 24576 candidates, few rows
+    (torch.float32, 130, 65536, 4096, 4, 4),     # 16384 fp32 candidates: 96 KiB
+    (torch.float32, 40, 32768, 2048, 2, 8),
+    (torch.int16, 130, 65536, 2560, 2, 8),       # 20480 candidates
+])
+def test_fused_rows_with_candidates_beyond_64_kib_of_lds(dtype, rows, n, k, j, k_mult):
+    g = torch.Generator().manual_seed(n + k + rows)
+    x = torch.randint(-2000, 2000, (rows, n), generator=g)
+    x = (x / 16).to(dtype) if dtype.is_floating_point else x.to(dtype)
+    _check(x, k, -1, j=j, k_mult=k_mult)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
 def test_fused_rows_special_values(dtype):
     g = torch.Generator().manual_seed(5)
