@@ -57,7 +57,7 @@ struct Geom {
   uint32_t chunks;       // > 1: one bucket per workgroup, scanned in that many chunks
   uint32_t groups;       // workgroups per row
   uint32_t slabs;        // > 1 (only with chunks > 1): workgroups sharing a bucket's chunks
-  uint32_t slab_chunks;  // chunks per slab; the last slab also takes the remainder
+  uint32_t slab_chunks;  // least chunks per slab: slab s takes chunks [s * chunks / slabs, (s + 1) * chunks / slabs)
 };
 
 // How a thread's queue holds values: in compare form (fast; no NaN may be
@@ -101,8 +101,10 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
   const uint32_t slab = g.slabs > 1 ? group % g.slabs : 0u;
   const uint32_t c0 = g.slabs > 1 ? group / g.slabs : group * per_group;
   // the chunks of this workgroup
-  const uint32_t it0 = slab * g.slab_chunks;
-  const uint32_t it1 = (g.slabs == 1 || slab + 1 == g.slabs) ? g.chunks : it0 + g.slab_chunks;
+  // (shared out evenly: with the remainder all on the last slab, 1024 chunks over
+  // 171 slabs left one workgroup 174 chunks and the others 5)
+  const uint32_t it0 = g.slabs == 1 ? 0u : (uint32_t)(((uint64_t)slab * g.chunks) / g.slabs);
+  const uint32_t it1 = g.slabs == 1 ? g.chunks : (uint32_t)(((uint64_t)(slab + 1) * g.chunks) / g.slabs);
   const uint32_t c = c0 + (t >> g.pieces_log2);
   const uint32_t piece = t & (pieces - 1);
   const bool has = c < g.b;

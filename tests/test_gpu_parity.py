@@ -457,6 +457,16 @@ def test_contiguous_buckets(rows, n, k, j, dtype):
     _check(x, k, -1, j=j, interleaved=False)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8])
+@pytest.mark.parametrize("rows,n,k,j,k_mult", [(2, 3024656, 4, 2, 1), (1, 5000011, 3, 1, 1), (3, 2000003, 2, 4, 4)])
+def test_contiguous_buckets_few_and_very_long(dtype, rows, n, k, j, k_mult):
+    # a bucket's chunks are shared out over many workgroups, unevenly when they do not divide
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randint(0, 200, (rows, n), generator=g).to(dtype) if dtype == torch.uint8 else \
+        (torch.randint(-100000, 100000, (rows, n), generator=g) / 64).to(dtype)
+    _check(x, k, -1, j=j, k_mult=k_mult, interleaved=False)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
 @pytest.mark.parametrize("n,k", [(40000, 16), (4100, 64), (100000, 2)])
 def test_contiguous_buckets_special_values(dtype, n, k):
