@@ -4,7 +4,7 @@
 //
 // One workgroup per row (stage2_radix_select.hip) pushes all of a row's
 // candidates through one CU: about 0.8 us per thousand candidates, 25 us at
-// 32768.  Here a row is cut into segments of kSegment candidates, one workgroup
+// 32768.  Here a row is cut into segments of 1024 or 4096 candidates, one workgroup
 // each, and up to four small kernels follow one another on the stream:
 //
 //   range:   every workgroup finds the smallest and largest order key of its
@@ -45,8 +45,12 @@ namespace regs = select::regs;
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / select::kWave;
-constexpr int kPerThread = 4;
-constexpr uint32_t kSegment = kThreads * kPerThread;  // candidates per workgroup
+// Candidates per thread of the chain's kernels (PT): 4, so that a few rows spread over
+// many CUs, or 16 when the rows are many enough for that anyway (a workgroup's fixed
+// work -- the row's histogram, the ranges, the search -- is then shared by four times
+// the candidates).  A segment is kThreads * PT candidates.
+constexpr int kPerThreadFew = 4, kPerThreadMany = 16;
+constexpr uint32_t kSoloSegment = 1024;  // the one-launch form's segments (one candidate per thread)
 constexpr uint32_t kListCap = 2048;                   // listed candidates a row can hold
 constexpr uint32_t kRankDirect = 256;                 // lists up to this size are ranked by counting
 
@@ -67,6 +71,7 @@ constexpr uint32_t kRangeCapacity = 4096;
 struct ChainPlan {
   bool use;
   bool solo;        // one launch does it (chain_solo_kernel)
+  int per_thread;   // candidates per thread of the chain's kernels
   uint32_t groups;  // workgroups per row
   uint32_t range_capacity;
   size_t range_off, hist_off, state_off, above_off, list_word_off, list_at_off, total;
@@ -74,33 +79,33 @@ struct ChainPlan {
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Thread t of a workgroup holds candidates first + u * kThreads, u = 0..kPerThread-1, of its row.
-template <typename E>
+// Thread t of a workgroup holds candidates first + u * kThreads, u = 0..PT-1, of its row.
+template <typename E, int PT>
 __device__ __forceinline__ void load_keys(const typename E::raw_t* __restrict__ cv, uint32_t first, uint32_t k0,
-                                          uint32_t (&key)[kPerThread], bool (&valid)[kPerThread]) {
-  typename E::raw_t raw[kPerThread];
+                                          uint32_t (&key)[PT], bool (&valid)[PT]) {
+  typename E::raw_t raw[PT];
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) {
+  for (int u = 0; u < PT; ++u) {
     valid[u] = first + u * kThreads < k0;
     raw[u] = valid[u] ? cv[first + u * kThreads] : (typename E::raw_t)0;
   }
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) key[u] = (uint32_t)E::key(raw[u]);
+  for (int u = 0; u < PT; ++u) key[u] = (uint32_t)E::key(raw[u]);
 }
 
-template <typename E>
+template <typename E, int PT>
 __global__ __launch_bounds__(kThreads) void chain_range_kernel(const typename E::raw_t* __restrict__ cand_values,
                                                                uint32_t k0, uint32_t groups, uint2* __restrict__ range,
                                                                uint32_t* __restrict__ hist, RowState* __restrict__ state) {
   __shared__ uint32_t wave_low[kWaves], wave_high[kWaves];
   const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
   const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
-  uint32_t key[kPerThread];
-  bool valid[kPerThread];
-  load_keys<E>(cand_values + (int64_t)row * k0, g * kSegment + tid, k0, key, valid);
+  uint32_t key[PT];
+  bool valid[PT];
+  load_keys<E, PT>(cand_values + (int64_t)row * k0, g * (kThreads * (uint32_t)PT) + tid, k0, key, valid);
   uint32_t low = ~0u, high = 0;
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) {
+  for (int u = 0; u < PT; ++u) {
     if (valid[u]) {
       low = key[u] < low ? key[u] : low;
       high = key[u] > high ? key[u] : high;
@@ -124,7 +129,7 @@ __global__ __launch_bounds__(kThreads) void chain_range_kernel(const typename E:
   }
 }
 
-template <typename E>
+template <typename E, int PT>
 __global__ __launch_bounds__(kThreads) void chain_hist_kernel(const typename E::raw_t* __restrict__ cand_values,
                                                               uint32_t k0, uint32_t groups,
                                                               const uint2* __restrict__ range, uint32_t entries,
@@ -133,14 +138,14 @@ __global__ __launch_bounds__(kThreads) void chain_hist_kernel(const typename E::
   __shared__ uint32_t red[2 * kWaves];
   const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
   const uint32_t tid = threadIdx.x;
-  uint32_t key[kPerThread];
-  bool valid[kPerThread];
-  load_keys<E>(cand_values + (int64_t)row * k0, g * kSegment + tid, k0, key, valid);
+  uint32_t key[PT];
+  bool valid[PT];
+  load_keys<E, PT>(cand_values + (int64_t)row * k0, g * (kThreads * (uint32_t)PT) + tid, k0, key, valid);
   for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = 0;
   uint32_t low, shift;
   regs::digit_of_row<kThreads>(range + (size_t)row * entries, entries, red, low, shift);  // (its barrier also covers the clearing)
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u)
+  for (int u = 0; u < PT; ++u)
     if (valid[u]) atomicAdd(&local[regs::hist_slot((key[u] - low) >> shift)], 1u);
   __syncthreads();
   uint32_t* h = hist + (size_t)row * regs::kHistWords;
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(kThreads) void chain_hist_kernel(const typename E::
   }
 }
 
-template <typename E>
+template <typename E, int PT>
 __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t groups, const uint2* __restrict__ range, uint32_t entries,
@@ -163,14 +168,14 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
   __shared__ uint32_t red[2 * kWaves];
   const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
   const uint32_t tid = threadIdx.x, lane = tid % select::kWave, wave = tid / select::kWave;
-  const uint32_t first = g * kSegment + tid;
+  const uint32_t first = g * (kThreads * (uint32_t)PT) + tid;
   // everything this workgroup reads is asked for at once: keys, indices, the row's histogram and ranges
-  uint32_t key[kPerThread], inv[kPerThread];
-  bool valid[kPerThread];
-  load_keys<E>(cand_values + (int64_t)row * k0, first, k0, key, valid);
+  uint32_t key[PT], inv[PT];
+  bool valid[PT];
+  load_keys<E, PT>(cand_values + (int64_t)row * k0, first, k0, key, valid);
   const int64_t* ci = cand_indices + (int64_t)row * k0;
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) inv[u] = valid[u] ? ~(uint32_t)ci[first + u * kThreads] : 0u;
+  for (int u = 0; u < PT; ++u) inv[u] = valid[u] ? ~(uint32_t)ci[first + u * kThreads] : 0u;
   const uint32_t* h = hist + (size_t)row * regs::kHistWords;
   for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = h[i];
   uint32_t low, shift;
@@ -182,10 +187,10 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
   __syncthreads();
   const regs::Found f = found;
   uint32_t mine = 0;
-  bool member[kPerThread];  // of a digit that is cut: ranked later, from the row's list
+  bool member[PT];  // of a digit that is cut: ranked later, from the row's list
   uint32_t listed = 0;
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) {
+  for (int u = 0; u < PT; ++u) {
     const uint32_t d = (key[u] - low) >> shift;
     // survivors known now: above B, and all of B when none of it is cut
     mine += (valid[u] && (d > f.digit || (d == f.digit && f.need == f.count))) ? 1u : 0u;
@@ -215,7 +220,7 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
 #pragma unroll
   for (int w = 0; w < kWaves; ++w) slot += (uint32_t)w < wave ? wave_listed[w] : 0u;
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) {
+  for (int u = 0; u < PT; ++u) {
     if (member[u]) {
       list_word[(size_t)row * k0 + slot] = ((uint64_t)key[u] << 32) | (uint64_t)inv[u];
       list_at[(size_t)row * k0 + slot] = first + u * kThreads;
@@ -224,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void chain_refine_kernel(
   }
 }
 
-template <typename E>
+template <typename E, int PT>
 __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t groups, int index_bits, const RowState* __restrict__ state,
@@ -236,7 +241,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
   __shared__ select::SharedT<2> sh;
   __shared__ uint64_t cut_word;
   __shared__ uint32_t listed_before;
-  __shared__ uint32_t wave_kept[kPerThread][kWaves];
+  __shared__ uint32_t wave_kept[PT][kWaves];
   __shared__ regs::Found found;
   __shared__ uint32_t lds_count;
   const uint32_t row = blockIdx.x / groups, g = blockIdx.x - row * groups;
@@ -310,15 +315,15 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
   const uint32_t n = cut_digit ? count : 0u;  // members ranked here, in LDS
   uint64_t* words = reinterpret_cast<uint64_t*>(dyn_lds);
   uint32_t* ats = reinterpret_cast<uint32_t*>(dyn_lds + (size_t)kListCap * sizeof(uint64_t));
-  const uint32_t first = g * kSegment + tid;
+  const uint32_t first = g * (kThreads * (uint32_t)PT) + tid;
   const raw_t* cv = cand_values + (int64_t)row * k0;
   const int64_t* ci = cand_indices + (int64_t)row * k0;
   // this thread's candidates: elements, keys and indices
-  raw_t raw[kPerThread];
-  uint32_t inv[kPerThread];
-  bool valid[kPerThread];
+  raw_t raw[PT];
+  uint32_t inv[PT];
+  bool valid[PT];
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) {
+  for (int u = 0; u < PT; ++u) {
     valid[u] = first + u * kThreads < k0;
     raw[u] = valid[u] ? cv[first + u * kThreads] : (raw_t)0;
     inv[u] = valid[u] ? ~(uint32_t)ci[first + u * kThreads] : 0u;
@@ -340,7 +345,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
       const uint32_t at = la[i];
       const uint32_t d = ((uint32_t)(w >> 32) - s.low) >> shift;
       if (d > digit || (d == digit && !cut_digit)) {
-        counted += at < g * kSegment ? 1u : 0u;
+        counted += at < g * (kThreads * (uint32_t)PT) ? 1u : 0u;
       } else if (d == digit) {
         const uint32_t slot = atomicAdd(&lds_count, 1u);
         words[slot] = w;
@@ -380,14 +385,14 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
     }
     // listed survivors of the segments before this one
     uint32_t before = 0;
-    for (uint32_t i = tid; i < n; i += kThreads) before += (ats[i] < g * kSegment && words[i] >= cut) ? 1u : 0u;
+    for (uint32_t i = tid; i < n; i += kThreads) before += (ats[i] < g * (kThreads * (uint32_t)PT) && words[i] >= cut) ? 1u : 0u;
     before = regs::wave_scan(before);
     if (lane == select::kWave - 1 && before != 0) atomicAdd(&listed_before, before);
   }
   // survivors of this thread, counted per u and wave (candidate order: u, then thread)
-  bool sel[kPerThread];
+  bool sel[PT];
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) {
+  for (int u = 0; u < PT; ++u) {
     const uint32_t key = (uint32_t)E::key(raw[u]);
     const uint32_t d = (key - s.low) >> shift;
     sel[u] = valid[u] && (d > digit || (d == digit && (((uint64_t)key << 32) | inv[u]) >= cut));
@@ -402,7 +407,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
   raw_t* ov = values + (int64_t)row * k;
   const int64_t oi = (int64_t)row * k;
 #pragma unroll
-  for (int u = 0; u < kPerThread; ++u) {
+  for (int u = 0; u < PT; ++u) {
     uint32_t o = base;
     for (int w = 0; w < kWaves; ++w) {
       if ((uint32_t)w < wave) o += wave_kept[u][w];
@@ -436,10 +441,10 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
 // from L2 for the most part.  The key ranges come from stage 1, or from the
 // keys themselves when stage 1 left none.
 // ---------------------------------------------------------------------------
-constexpr int kSoloThreads = 1024;  // == kSegment
+constexpr int kSoloThreads = 1024;  // == kSoloSegment
 constexpr int kSoloWaves = kSoloThreads / select::kWave;
 constexpr uint32_t kSoloRankDirect = 512;
-static_assert((uint32_t)kSoloThreads == kSegment, "a thread's u-th candidate lies in segment u");
+static_assert((uint32_t)kSoloThreads == kSoloSegment, "a thread's u-th candidate lies in segment u");
 
 template <typename E, int NPT, bool OWN_RANGE>
 __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
@@ -649,23 +654,32 @@ constexpr int64_t kSoloMaxWorkgroups = 256;
 // is what bounds them, keys of at most 32 bits and indices below 2^31.  Measured,
 // select alone, microseconds, fp16 / fp32, chain against one workgroup per row:
 // 16 rows of 16384: 14.6 / 18.9 against 16.3 / 18.3; 32 rows of 16384: 21.7 / 35.2;
-// 16 rows of 65536: 34 / 33 against 70 / 73; 32 rows of 65536: 52 / 49;
-// 64 rows of 65536: 92 / 89; 32 rows of 131072: 119 / 125 against 121 / 125.
+// 17-32 rows of 32768: 29 / 38 against 23 / 26; 16 rows of 65536: 34 / 33 against
+// 70 / 73; 64 rows of 49152: 43 / 46 against 54 / 58, 96 rows 59 / 62 against 56 / 72;
+// 64 rows of 65536: 49 / 53 against 72 / 74, 96 rows 79 / 84 against 74 / 75;
+// 64 rows of 131072: 99 / 110 against 107 / 118, 96 rows 141 / 162 against 142 / 173.
+// Segments of 4096 candidates from 1024 workgroups of the short ones on: 32 rows of
+// 131072 took 120 / 127 us with segments of 1024, 33 rows 65 / 71 us with 4096.
 constexpr int64_t kChainMinCandidates = 10240;  // (8192: 11.8 us against 10.5 for one workgroup)
 constexpr int64_t kChainMaxCandidates = 1 << 17;
 constexpr int64_t kChainMaxRows = 16;
-constexpr int64_t kChainMaxRowsLong = 32;  // rows of kChainLong candidates and more
-constexpr int64_t kChainLong = 1 << 16;
+constexpr int64_t kChainMaxRowsLong = 64;  // rows of more than kSoloMaxCandidates candidates
+constexpr int64_t kChainShortSegmentGroups = 1024;
 
 ChainPlan plan_chain(int64_t rows, int64_t k0, int64_t k, int64_t index_bound, int dtype) {
   ChainPlan pl{};
   pl.use = false;
   const int es = elem_bytes(dtype);
   if (es == 0 || es > 4 || rows <= 0 || k <= 0 || k >= k0) return pl;
-  if (rows > (k0 >= kChainLong ? kChainMaxRowsLong : kChainMaxRows)) return pl;
   if (k0 < kChainMinCandidates || k0 > kChainMaxCandidates || index_bound > 0x7fffffffll) return pl;
-  pl.groups = (uint32_t)((k0 + kSegment - 1) / kSegment);
+  if (rows > (k0 > kSoloMaxCandidates ? kChainMaxRowsLong : kChainMaxRows)) return pl;
+  pl.groups = (uint32_t)((k0 + kSoloSegment - 1) / kSoloSegment);
+  pl.per_thread = rows * (int64_t)pl.groups > kChainShortSegmentGroups ? kPerThreadMany : kPerThreadFew;
   pl.solo = k0 <= kSoloMaxCandidates && rows * (int64_t)pl.groups <= kSoloMaxWorkgroups;
+  if (!pl.solo) {
+    const int64_t segment = (int64_t)kThreads * pl.per_thread;
+    pl.groups = (uint32_t)((k0 + segment - 1) / segment);
+  }
   pl.range_off = 0;
   pl.range_capacity = pl.groups > kRangeCapacity ? pl.groups : kRangeCapacity;
   pl.hist_off = align_up((size_t)rows * pl.range_capacity * sizeof(uint2), 256);
@@ -698,11 +712,8 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
     const dim3 grid((unsigned)(rows * pl.groups)), block(kThreads);
     const size_t emit_lds = (size_t)kListCap * (sizeof(uint64_t) + sizeof(uint32_t));
     uint32_t entries = range_entries;
-    if (entries == 0 && !pl.solo) {  // stage 1 left no key ranges
-      hipLaunchKernelGGL((chain_range_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups, range, hist,
-                         state);
-      entries = pl.groups;
-    }
+    const bool own_ranges = entries == 0 && !pl.solo;  // stage 1 left no key ranges
+    if (own_ranges) entries = pl.groups;
     if (pl.solo) {
       const size_t solo_lds = (size_t)(kListCap + 8) * (sizeof(uint64_t) + sizeof(uint32_t));
       const dim3 solo_block(kSoloThreads);
@@ -722,15 +733,24 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
 #undef ATK_SOLO
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }
-    if (!hist_done || range_entries == 0)
-      hipLaunchKernelGGL((chain_hist_kernel<E>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups,
-                         (const uint2*)range, entries, hist);
-    hipLaunchKernelGGL((chain_refine_kernel<E>), grid, block, 0, stream, cv, cand_indices, (uint32_t)k0, (uint32_t)k,
-                       pl.groups, (const uint2*)range, entries, (const uint32_t*)hist, state, above, list_word,
-                       list_at);
-    hipLaunchKernelGGL((chain_emit_kernel<E>), grid, block, emit_lds, stream, cv, cand_indices, (uint32_t)k0,
-                       (uint32_t)k, pl.groups, index_bits, (const RowState*)state, (const uint32_t*)above,
-                       (const uint64_t*)list_word, (const uint32_t*)list_at, static_cast<raw_t*>(values), indices);
+#define ATK_CHAIN(PT)                                                                                              \
+  {                                                                                                                \
+    if (own_ranges)                                                                                                \
+      hipLaunchKernelGGL((chain_range_kernel<E, PT>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups, range,  \
+                         hist, state);                                                                             \
+    if (!hist_done || range_entries == 0)                                                                          \
+      hipLaunchKernelGGL((chain_hist_kernel<E, PT>), grid, block, 0, stream, cv, (uint32_t)k0, pl.groups,          \
+                         (const uint2*)range, entries, hist);                                                      \
+    hipLaunchKernelGGL((chain_refine_kernel<E, PT>), grid, block, 0, stream, cv, cand_indices, (uint32_t)k0,       \
+                       (uint32_t)k, pl.groups, (const uint2*)range, entries, (const uint32_t*)hist, state, above,  \
+                       list_word, list_at);                                                                        \
+    hipLaunchKernelGGL((chain_emit_kernel<E, PT>), grid, block, emit_lds, stream, cv, cand_indices, (uint32_t)k0,  \
+                       (uint32_t)k, pl.groups, index_bits, (const RowState*)state, (const uint32_t*)above,         \
+                       (const uint64_t*)list_word, (const uint32_t*)list_at, static_cast<raw_t*>(values),          \
+                       indices);                                                                                   \
+  }
+    if (pl.per_thread == kPerThreadMany) ATK_CHAIN(kPerThreadMany) else ATK_CHAIN(kPerThreadFew)
+#undef ATK_CHAIN
     return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
   } else {
     (void)pl; (void)cand_values; (void)cand_indices; (void)rows; (void)k0; (void)k; (void)index_bits; (void)values;
@@ -758,7 +778,7 @@ bool describe_chain_select(int64_t rows, int64_t k0, int64_t k, int64_t index_bo
   out += "[chain_range_kernel<" + t + "> + chain_hist_kernel<" + t +
          "> unless stage 1 left key ranges and histogram] + chain_refine_kernel<" + t +
          "> + chain_emit_kernel<" + t + "> grid=" + std::to_string(rows * (int64_t)pl.groups) + " block=" +
-         std::to_string(kThreads);
+         std::to_string(kThreads) + " per_thread=" + std::to_string(pl.per_thread);
   return true;
 }
 

@@ -152,6 +152,14 @@ def test_chain_select_narrows_a_crowded_digit(dtype, k0, k):
     _chain_case(["outliers", "crowded", "tied outliers", "spread"], k0, k, dtype, seed=k0 * 3 + k)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int32])
+@pytest.mark.parametrize("k0,k", [(49153, 30000), (65536, 777), (131072, 5000), (33000, 32999)])
+def test_chain_select_with_long_segments(dtype, k0, k):
+    # 40 rows of more than 32768 candidates: the chain's workgroups take 4096 candidates each
+    kinds = ["spread", "ties", "equal", "steps", "outliers", "crowded", "tied outliers", "spread"] * 5
+    _chain_case(kinds, k0, k, dtype, seed=k0 + k + 1)
+
+
 def test_chain_select_needs_no_cut_when_the_digit_belongs_whole():
     # k falls exactly on a boundary between two values: every member of the cut digit survives
     k0 = 16384

@@ -101,8 +101,11 @@ def test_describe_names_the_planned_kernels():
     assert describe(64, 1024, 1, 8, 1, 2).startswith("fused_regs_kernel<f16, J=1")
     # the select over several workgroups per row: few rows only, one launch up to 32768 candidates
     assert "chain_solo_kernel<f32> grid=16 " in describe(1, 1 << 24, 0, 8192, 2, 2)
-    assert "chain_emit_kernel<f32> grid=512 " in describe(8, 1 << 22, 0, 32768, 2, 2)
-    assert "chain_" not in describe(64, 1 << 18, 0, 16384, 2, 8)
+    assert "chain_emit_kernel<f32> grid=512 block=256 per_thread=4" in describe(8, 1 << 22, 0, 32768, 2, 2)
+    # more rows of more than 32768 candidates: segments of 4096 candidates; beyond 64 rows other selects
+    assert "chain_emit_kernel<f32> grid=2048 block=256 per_thread=16" in describe(64, 1 << 18, 0, 16384, 2, 8)
+    assert "chain_" not in describe(65, 1 << 18, 0, 16384, 2, 8)
+    assert "chain_" not in describe(17, 1 << 20, 0, 16384, 1, 2)
     # a misaligned input: scalar loads, and two kernels instead of the fused one
     odd = describe(1024, 32768, 1, 2048, 4, 4, x=4098)
     assert odd.startswith("stream_kernel<f16, J=4, V=1") and "select_kernel<f16" in odd
