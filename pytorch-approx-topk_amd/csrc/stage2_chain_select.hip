@@ -26,11 +26,12 @@
 // When the digit B holds more candidates than a workgroup's LDS list takes
 // (kListCap; keys that crowd into a small part of their span: heavy tails,
 // outliers), the members of B are counted again by the next 11 bits of their
-// offsets, and so on until the cut digit fits or no bits are left (every emit
-// workgroup does this over the row's list in global memory, which holds all of
-// B).  Only a row with more than kListCap candidates of one and the same key
-// around the cut is selected by its first workgroup alone, with the block-wide
-// radix select over all of its candidates.  When stage 1 ends in kernels that can leave key ranges and the
+// offsets, and so on, through the bits of the key and then of the index, until
+// the cut digit fits (every emit workgroup does this over the row's list in
+// global memory, which holds all of B; the one-launch form narrows over the key
+// bits and leaves a row with more than kListCap candidates of one key around
+// the cut to its first workgroup, with the block-wide radix select over all of
+// its candidates).  When stage 1 ends in kernels that can leave key ranges and the
 // histogram behind (KeyRangeOut: the streaming kernel's slabs and their merge),
 // the range and hist launches are skipped.  Results are those of the
 // one-workgroup kernel: same survivors, same order.
@@ -255,12 +256,20 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
   uint32_t counted = 0;
   for (uint32_t p = tid; p < g; p += kThreads) counted += above[(size_t)row * groups + p];
   const RowState s = state[row];
-  uint32_t digit = s.digit, shift = s.shift, need = s.need, count = s.count;
+  // A candidate's word less the row's smallest key, (key - low, inverted index), is what the
+  // digits are taken from: the first 32 bits are the key's offset, the rest the index, so that
+  // candidates of one key are told apart by their indices when the digits reach that far.
+  const uint64_t low_word = (uint64_t)s.low << 32;
+  uint64_t digit = s.digit;  // of (word - low_word) >> shift
+  uint32_t shift = s.shift + 32u, need = s.need, count = s.count;
   const uint32_t listed = need != count ? count : 0u;  // entries of the row's list: all members of B
-  if (listed > kListCap) {
+  const bool narrowed = listed > kListCap;
+  if (narrowed) {
     // More members than a workgroup ranks: they are counted again by the next bits of their
-    // offsets, which narrows the digit that is cut, until its members fit (the histogram borrows
-    // the memory of the LDS list, which is filled afterwards).
+    // words, which narrows the digit that is cut, until its members fit (the histogram borrows
+    // the memory of the LDS list, which is filled afterwards).  Every workgroup of the row goes
+    // through the whole list once per level; even for a row of 131072 equal keys that is several
+    // times faster than leaving the row to one workgroup (65536 equal keys: 460 us there).
     uint32_t* local = reinterpret_cast<uint32_t*>(dyn_lds);
     while (need != count && count > kListCap && shift != 0) {
       const uint32_t finer = shift > (uint32_t)regs::kDigitBits ? shift - (uint32_t)regs::kDigitBits : 0u;
@@ -268,8 +277,8 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
       for (uint32_t i = tid; i < regs::kHistWords; i += kThreads) local[i] = 0;
       __syncthreads();
       for (uint32_t i = tid; i < listed; i += kThreads) {
-        const uint32_t off = (uint32_t)(lw[i] >> 32) - s.low;
-        if ((off >> shift) == digit) atomicAdd(&local[regs::hist_slot((off >> finer) & mask)], 1u);
+        const uint64_t off = lw[i] - low_word;
+        if ((off >> shift) == digit) atomicAdd(&local[regs::hist_slot((uint32_t)(off >> finer) & mask)], 1u);
       }
       __syncthreads();
       if (wave == 0) {
@@ -278,17 +287,18 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
       }
       __syncthreads();
       const regs::Found f = found;
-      digit = (digit << (shift - finer)) | f.digit;
+      digit = (digit << (shift - finer)) | (uint64_t)f.digit;
       shift = finer;
       need = f.need;
       count = f.count;
     }
   }
   if (need != count && count > kListCap) {
-    // More than kListCap candidates of one key around the cut: the row's first
-    // workgroup runs the block-wide radix select of stage2_select.h over all of
-    // the row's candidates, read from global memory (slow, for rows with
-    // thousands of equal keys only).
+    // No bits left and still more than the list takes: thousands of candidates
+    // with one key and one index, which only a caller of the stand-alone select
+    // can hand over (stage 1 gives every candidate its own index).  The row's
+    // first workgroup runs the block-wide radix select of stage2_select.h over
+    // all of the row's candidates, read from global memory.
     if (g != 0) return;
     const raw_t* rv = cand_values + (int64_t)row * k0;
     const int64_t* ri = cand_indices + (int64_t)row * k0;
@@ -343,7 +353,7 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
     for (uint32_t i = tid; i < listed; i += kThreads) {
       const uint64_t w = lw[i];
       const uint32_t at = la[i];
-      const uint32_t d = ((uint32_t)(w >> 32) - s.low) >> shift;
+      const uint64_t d = (w - low_word) >> shift;
       if (d > digit || (d == digit && !cut_digit)) {
         counted += at < g * (kThreads * (uint32_t)PT) ? 1u : 0u;
       } else if (d == digit) {
@@ -394,8 +404,14 @@ __global__ __launch_bounds__(kThreads) void chain_emit_kernel(
 #pragma unroll
   for (int u = 0; u < PT; ++u) {
     const uint32_t key = (uint32_t)E::key(raw[u]);
-    const uint32_t d = (key - s.low) >> shift;
-    sel[u] = valid[u] && (d > digit || (d == digit && (((uint64_t)key << 32) | inv[u]) >= cut));
+    const uint64_t word = ((uint64_t)key << 32) | inv[u];
+    if (!narrowed) {  // the digit lies within the key
+      const uint32_t d = (key - s.low) >> (shift - 32u);
+      sel[u] = valid[u] && (d > (uint32_t)digit || (d == (uint32_t)digit && word >= cut));
+    } else {
+      const uint64_t d = (word - low_word) >> shift;
+      sel[u] = valid[u] && (d > digit || (d == digit && word >= cut));
+    }
     const uint64_t m = __ballot(sel[u]);
     if (lane == 0) wave_kept[u][wave] = (uint32_t)__popcll(m);
   }

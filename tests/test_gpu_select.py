@@ -160,6 +160,20 @@ def test_chain_select_with_long_segments(dtype, k0, k):
     _chain_case(kinds, k0, k, dtype, seed=k0 + k + 1)
 
 
+@pytest.mark.parametrize("k0", [20000, 40000, 70000])
+def test_chain_select_of_identical_candidates(k0):
+    # only a caller of the stand-alone select can hand over candidates that share key and index:
+    # no bit tells them apart, and the row goes to the whole-row path; any k of them are the answer
+    cv = torch.full((2, k0), 2.0)
+    cv[1, : k0 // 2] = 5.0
+    ci = torch.full((2, k0), 7, dtype=torch.int64)
+    k = k0 // 2 + 1234
+    v, i = _select(cv, ci, k, 1 << 20)
+    assert torch.equal(i.cpu(), torch.full((2, k), 7, dtype=torch.int64))
+    assert torch.equal(v[0].cpu(), torch.full((k,), 2.0))
+    assert torch.equal(v[1].cpu(), torch.cat([torch.full((k0 // 2,), 5.0), torch.full((1234,), 2.0)]))
+
+
 def test_chain_select_needs_no_cut_when_the_digit_belongs_whole():
     # k falls exactly on a boundary between two values: every member of the cut digit survives
     k0 = 16384
