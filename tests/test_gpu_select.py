@@ -65,8 +65,15 @@ def test_select_all_equal_and_wide_indices():
     assert_same(v, i, ev, ei, "all-equal rows")
 
 
-def test_select_under_graph_replay():
-    cv, ci = _candidates(2, 150000, torch.float32, 11, True, 1 << 21)
+@pytest.mark.parametrize("rows,k0", [
+    (2, 150000),     # passes over many workgroups
+    (2, 70000),      # the chain of launches, ties told apart by index (row state and list counters in the workspace)
+    (40, 40000),     # the chain with long segments
+    (3, 20000),      # the one-launch form
+    (70, 40000),     # one workgroup per row
+])
+def test_select_under_graph_replay(rows, k0):
+    cv, ci = _candidates(rows, k0, torch.float32, 11 + rows, True, 1 << 21)
     from approx_topk import _native
     cvg, cig = cv.cuda(), ci.cuda()
     _native.select(cvg, cig, 5000, 1 << 21)
@@ -77,9 +84,10 @@ def test_select_under_graph_replay():
     ev, ei = oracle.stage2(cv, ci, 5000)
     for _ in range(3):
         v.zero_(); i.zero_()
+        _native.select(cvg, cig, 77, 1 << 21)    # eager work between the replays
         graph.replay()
         torch.cuda.synchronize()
-        assert_same(v, i, ev, ei, "graph replay")
+        assert_same(v, i, ev, ei, f"graph replay rows={rows} k0={k0}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
