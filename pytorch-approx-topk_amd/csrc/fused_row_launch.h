@@ -9,7 +9,9 @@ namespace fused {
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
 static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                          uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
-  if (pl.in_registers) {
+  if constexpr (MAXW > 8) {
+    if (pl.in_registers) return ATK_ERR_ARG;  // (the register kernel is built for eight waves)
+  } else if (pl.in_registers) {
     auto kern = fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED>;
     if (pl.lds_bytes > 48 * 1024) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -47,7 +49,10 @@ static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, 
 template <typename E, int J, int VF>
 static int launch_v(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                     uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
-  if (pl.waves > 8) return ATK_ERR_ARG;  // the planner never asks for more
+  if (pl.waves > 16) return ATK_ERR_ARG;  // the planner never asks for more
+  if (pl.waves > 8)  // candidates beyond the usual LDS budget: one workgroup of sixteen waves per CU
+    return pl.pos16 ? launch_one<E, J, VF, 16, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
+                    : launch_one<E, J, VF, 16, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
   return pl.pos16 ? launch_one<E, J, VF, 8, uint16_t>(pl, x, rows, g, k0, k, values, indices, stream)
                   : launch_one<E, J, VF, 8, uint32_t>(pl, x, rows, g, k0, k, values, indices, stream);
 }

@@ -15,14 +15,14 @@ constexpr size_t kSoloRow = 256 * 1024;
 // Dynamic LDS a workgroup may use (candidates + hand-over); the select's own
 // block adds about 9 KiB.
 constexpr size_t kLdsBudget = 64 * 1024;
-// For rows of up to 256 KiB the candidates may take twice that (one workgroup
-// per CU then): the alternative parks them in HBM and selects with one
-// workgroup per row as well.  Measured with the larger budget: fp16 [256, 65536]
-// k0=32768 71 -> 52 us, [1024, 65536] 312 -> 196 us, fp32 [256, 65536] k0=16384
-// 52 -> 39 us; longer rows lose (fp16 [128, 2^20] k0=32768 87 -> 115 us, fp32
-// [1024, 131072] k0=16384 195 -> 208 us).
-constexpr size_t kLdsBudgetShortRows = 128 * 1024;
-constexpr size_t kShortRowsForLds = 256 * 1024;
+// The candidates may take twice that, one workgroup of sixteen waves per CU
+// then: the alternative parks them in HBM and selects with one workgroup per
+// row as well.  Measured against the two-kernel path: fp16 [256, 65536]
+// k0=32768 71 -> 38 us, [1024, 65536] 312 -> 142 us, [512, 262144] 184 -> 113 us,
+// [128, 2^20] 90 -> 85 us, fp32 [256, 65536] k0=16384 52 -> 35 us, [2048, 131072]
+// 375 -> 336 us.  (With eight waves the larger budget lost for rows beyond
+// 256 KiB: [128, 2^20] 87 -> 115 us.)
+constexpr size_t kLdsBudgetLarge = 128 * 1024;
 // Most waves per workgroup.  Measured over shapes from [4096, 4096] to
 // [256, 65536]: 8 beats 16 (more workgroups per CU, in different phases, and
 // cheaper barriers) and is never far behind 4.
@@ -98,9 +98,12 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   const int skey = (dtype == ATK_U8 || dtype == ATK_I8) ? 2 : es;  // stored key width
   const size_t cand_bytes = (((size_t)k0 * skey + 15) & ~(size_t)15) +
                             (((size_t)k0 * (pl.pos16 ? 2 : 4) + 15) & ~(size_t)15);
-  const size_t lds_budget = row_bytes <= kShortRowsForLds ? kLdsBudgetShortRows : kLdsBudget;
+  const size_t lds_budget = kLdsBudgetLarge;
   if (cand_bytes > lds_budget) return pl;
 
+  // With more than the usual LDS budget taken, one workgroup has the CU to itself:
+  // sixteen waves then (the scan and the selection both gain from them).
+  const uint32_t max_waves = cand_bytes > kLdsBudget ? 2 * kMaxWaves : kMaxWaves;
   // Waves sharing a tile: as many as keep each share at least max(j, 8)
   // sub-rows long, the workgroup within its wave limit and LDS within budget.
   // When all tiles are in flight at once the hand-over area may lie on top of
@@ -108,29 +111,29 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   const int cmp_size = es > 4 ? 8 : 4;
   const int64_t min_run = j > 8 ? j : 8;
   auto hand_bytes = [&](uint32_t split) {
-    const uint32_t waves = pl.tiles * split <= kMaxWaves ? pl.tiles * split : kMaxWaves;
+    const uint32_t waves = pl.tiles * split <= max_waves ? pl.tiles * split : max_waves;
     return (size_t)(waves - waves / split) * pl.vec * j * stream::kWave * (cmp_size + 4);
   };
   auto lds_need = [&](uint32_t split) {
-    const bool one_round = pl.tiles * split <= kMaxWaves;
+    const bool one_round = pl.tiles * split <= max_waves;
     const size_t hand = hand_bytes(split);
     return one_round ? (hand > cand_bytes ? hand : cand_bytes) : cand_bytes + hand;
   };
   uint32_t split = 1;
-  if (pl.tiles < kMaxWaves) {
-    for (uint32_t cand = 2; cand * pl.tiles <= kMaxWaves; cand *= 2) {
+  if (pl.tiles < max_waves) {
+    for (uint32_t cand = 2; cand * pl.tiles <= max_waves; cand *= 2) {
       if (full / cand < min_run || lds_need(cand) > lds_budget) break;
       split = cand;
     }
   }
   pl.split = split;
-  pl.waves = pl.tiles * split <= kMaxWaves ? pl.tiles * split : kMaxWaves;
-  const bool one_round = pl.tiles * split <= kMaxWaves;
+  pl.waves = pl.tiles * split <= max_waves ? pl.tiles * split : max_waves;
+  const bool one_round = pl.tiles * split <= max_waves;
   pl.hand_off = (split > 1 && !one_round) ? (uint32_t)cand_bytes : 0u;
   pl.lds_bytes = lds_need(split);
   // every tile has its waves: stage 2 runs on the candidates where they are, in
   // registers, and needs the histogram's room in LDS
-  pl.in_registers = one_round;
+  pl.in_registers = one_round && pl.waves <= kMaxWaves;  // (the register kernel is built for eight waves)
   if (pl.in_registers && pl.lds_bytes < regs::kLdsBytes) pl.lds_bytes = regs::kLdsBytes;
   // survivors staged in LDS, eight bytes each (element, 32-bit index), when that fits
   pl.staged = pl.in_registers && pl.pos16 && es <= 4 && (size_t)k * 8 <= kLdsBudget;
