@@ -101,9 +101,13 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   const size_t lds_budget = kLdsBudgetLarge;
   if (cand_bytes > lds_budget) return pl;
 
-  // With more than the usual LDS budget taken, one workgroup has the CU to itself:
-  // sixteen waves then (the scan and the selection both gain from them).
-  const uint32_t max_waves = cand_bytes > kLdsBudget ? 2 * kMaxWaves : kMaxWaves;
+  // With more than the usual LDS budget taken, or with no more rows than CUs, one
+  // workgroup has the CU to itself: sixteen waves then, when eight would go through
+  // the tiles in several rounds (the scan and the selection both gain: fp16
+  // [256, 65536] k0=16384 32.8 -> 25.8 us, [200, 32768] k0=16384 30.3 -> 22.7 us; with
+  // 300-512 rows eight waves stay ahead, 43 against 49 us at [512, 65536]).
+  const uint32_t max_waves =
+      (cand_bytes > kLdsBudget || (rows <= kAllCus && pl.tiles > kMaxWaves)) ? 2 * kMaxWaves : kMaxWaves;
   // Waves sharing a tile: as many as keep each share at least max(j, 8)
   // sub-rows long, the workgroup within its wave limit and LDS within budget.
   // When all tiles are in flight at once the hand-over area may lie on top of
