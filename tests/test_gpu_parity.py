@@ -286,6 +286,9 @@ def test_fused_rows_shapes(n, k, j, k_mult):
     (torch.float32, 130, 65536, 4096, 4, 4),     # 16384 fp32 candidates: 96 KiB
     (torch.float32, 40, 32768, 2048, 2, 8),
     (torch.int16, 130, 65536, 2560, 2, 8),       # 20480 candidates
+    (torch.float32, 300, 16384, 1024, 2, 8),     # more rows than CUs: eight waves, the tiles in two rounds
+    (torch.float16, 300, 32768, 2048, 1, 8),
+    (torch.float16, 256, 32768, 2048, 1, 8),     # no more rows than CUs: sixteen waves
 ])
 def test_fused_rows_with_candidates_beyond_64_kib_of_lds(dtype, rows, n, k, j, k_mult):
     g = torch.Generator().manual_seed(n + k + rows)
