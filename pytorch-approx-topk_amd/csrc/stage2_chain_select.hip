@@ -462,7 +462,7 @@ constexpr int kSoloWaves = kSoloThreads / select::kWave;
 constexpr uint32_t kSoloRankDirect = 512;
 static_assert((uint32_t)kSoloThreads == kSoloSegment, "a thread's u-th candidate lies in segment u");
 
-template <typename E, int NPT, bool OWN_RANGE>
+template <typename E, int NPT, bool OWN_RANGE, bool TIES = (sizeof(typename E::raw_t) == 1)>
 __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t groups, int index_bits, const uint2* __restrict__ range, uint32_t entries,
@@ -551,11 +551,101 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     shift = finer;
   }
   const bool cut_digit = f.need != f.count;  // else every member of B survives
-  if (cut_digit && f.count > kListCap) {
-    // More than kListCap candidates of one key around the cut: the row's first
-    // workgroup runs the block-wide radix select of stage2_select.h over all of
-    // the row's candidates, read from global memory (slow, for rows with
-    // thousands of equal keys only).
+  // TIES: shift == 0 and still too many -- thousands of candidates of one key around the cut,
+  // which is what stage 1 makes of saturated 8-bit data (the bucket maxima of uniform uint8 are
+  // all 255) -- and their indices decide.  Built for the 1-byte types only: the code costs the
+  // kernel 4-5 us whether it runs or not (it sits at its register limit).
+  const bool tie_mode = TIES && cut_digit && f.count > kListCap;
+  const uint32_t own = g * kSoloThreads + tid;  // this thread's candidate of segment g
+  const bool own_valid = own < k0;
+  // survivors above the cut digit (or in it, when it belongs whole) in the
+  // segments before this one, and the members of a cut digit: listed, or flagged for the
+  // look at their indices below
+  uint32_t before = 0;
+  uint32_t own_key = 0;
+  [[maybe_unused]] uint32_t members = 0;
+#pragma unroll
+  for (int u = 0; u < NPT; ++u) {
+    const uint32_t d = (key[u] - low) >> shift;
+    const bool ok = valid(u);
+    if ((uint32_t)u < g) before += (ok && (d > f.digit || (d == f.digit && !cut_digit))) ? 1u : 0u;
+    if ((uint32_t)u == g) own_key = key[u];
+    if (ok && cut_digit && d == f.digit) {
+      if constexpr (TIES) members |= 1u << u;
+      if (!tie_mode) {
+        const uint32_t at = (uint32_t)u * kSoloThreads + tid;
+        const uint32_t slot = atomicAdd(&list_count, 1u);
+        words[slot] = (uint64_t)key[u] << 32;  // (the index follows below, for all members in one trip to memory)
+        ats[slot] = at;
+      }
+    }
+  }
+  uint32_t need = f.need, count = f.count;
+  uint64_t floor_word = 0;  // tie mode, when a whole group of indices survives: its smallest word
+  if constexpr (TIES) {
+    if (tie_mode) {
+      // The members (all of one key) are counted by the leading bits of their inverted indices,
+      // 11 at a time, until the group that is cut fits the list.  Their indices are read eight
+      // segments at a time (the low halves: the planner sends only indices below 2^31 here).
+      const uint32_t* ci_low = reinterpret_cast<const uint32_t*>(ci);
+      auto for_members = [&](auto&& fn) __attribute__((always_inline)) {
+        constexpr int kChunk = NPT < 8 ? NPT : 8;
+#pragma unroll
+        for (int c0 = 0; c0 < NPT; c0 += kChunk) {
+          uint32_t iv[kChunk];
+#pragma unroll
+          for (int e = 0; e < kChunk; ++e) {
+            const uint32_t i = (uint32_t)(c0 + e) * kSoloThreads + tid;
+            iv[e] = i < k0 ? ci_low[2u * i] : 0u;
+          }
+#pragma unroll
+          for (int e = 0; e < kChunk; ++e)
+            if ((members >> (c0 + e)) & 1u) fn((uint32_t)(c0 + e), ~iv[e]);
+        }
+      };
+      uint32_t ishift = 32, iprefix = 0;  // the group: inverted indices whose bits from ishift up are iprefix
+      while (need != count && count > kListCap && ishift != 0) {
+        const uint32_t finer = ishift > (uint32_t)regs::kDigitBits ? ishift - (uint32_t)regs::kDigitBits : 0u;
+        const uint32_t mask = (1u << (ishift - finer)) - 1u;
+        __syncthreads();  // everyone has read `found`, wave 0 the histogram
+        for (uint32_t i = tid; i < (uint32_t)regs::kBins; i += kSoloThreads) hist[i] = 0;
+        __syncthreads();
+        for_members([&](uint32_t, uint32_t inv) {
+          if (ishift == 32u || (inv >> ishift) == iprefix) atomicAdd(&hist[(inv >> finer) & mask], 1u);
+        });
+        __syncthreads();
+        if (wave == 0) {
+          const regs::Found f2 = regs::find_bin_wave<false>(hist, need, count, lane);
+          if (lane == 0) found = f2;
+        }
+        __syncthreads();
+        const regs::Found f2 = found;
+        iprefix = (iprefix << (ishift - finer)) | f2.digit;
+        ishift = finer;
+        need = f2.need;
+        count = f2.count;
+      }
+      if (ishift != 32u && (need == count || count <= kListCap)) {
+        const uint64_t key_word = (uint64_t)(low + f.digit) << 32;  // (shift == 0: the digit is the key's offset)
+        for_members([&](uint32_t u, uint32_t inv) {
+          const uint32_t group = inv >> ishift;
+          if (group > iprefix || (group == iprefix && need == count)) {
+            before += u < g ? 1u : 0u;  // survives whatever the list says
+          } else if (group == iprefix) {
+            const uint32_t slot = atomicAdd(&list_count, 1u);
+            words[slot] = key_word | (uint64_t)inv;
+            ats[slot] = u * kSoloThreads + tid;
+          }
+        });
+        if (need == count) floor_word = key_word | ((uint64_t)iprefix << ishift);
+      }
+    }
+  }
+  if (need != count && count > kListCap) {
+    // More than kListCap candidates of one key around the cut (TIES: of one key and
+    // one index, which only a caller of the stand-alone select can hand over): the
+    // row's first workgroup runs the block-wide radix select of stage2_select.h over
+    // all of the row's candidates, read from global memory.
     if (g != 0) return;
     auto key_at = [&](uint32_t i) -> key_t { return E::key(cv[i]); };
     auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)ci[i]; };
@@ -576,26 +666,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
         });
     return;
   }
-  const uint32_t own = g * kSoloThreads + tid;  // this thread's candidate of segment g
-  const bool own_valid = own < k0;
-  // survivors above the cut digit (or in it, when it belongs whole) in the
-  // segments before this one, and the members of a cut digit listed
-  uint32_t before = 0;
-  uint32_t own_key = 0;
-#pragma unroll
-  for (int u = 0; u < NPT; ++u) {
-    const uint32_t d = (key[u] - low) >> shift;
-    const bool ok = valid(u);
-    if ((uint32_t)u < g) before += (ok && (d > f.digit || (d == f.digit && !cut_digit))) ? 1u : 0u;
-    if ((uint32_t)u == g) own_key = key[u];
-    if (ok && cut_digit && d == f.digit) {
-      const uint32_t at = (uint32_t)u * kSoloThreads + tid;
-      const uint32_t slot = atomicAdd(&list_count, 1u);
-      words[slot] = (uint64_t)key[u] << 32;  // (the index follows below, for all members in one trip to memory)
-      ats[slot] = at;
-    }
-  }
-  const uint32_t n = cut_digit ? f.count : 0u;  // (== list_count after the barrier)
+  const uint32_t n = need != count ? count : 0u;  // (== list_count after the barrier)
   if (tid < 8u) {  // entries past the list's end beat nothing (ranking reads it in groups of eight)
     words[n + tid] = 0ull;
     ats[n + tid] = ~0u;
@@ -606,9 +677,10 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   // the index load made the kernel 5 us slower, measured.)
   const raw_t own_raw = own_valid ? cv[own] : (raw_t)0;
   const uint32_t own_inv = own_valid ? ~(uint32_t)ci[own] : 0u;
-  uint64_t cut = 0;  // the weakest surviving member of B (0: all of them survive)
+  uint64_t cut = floor_word;  // the weakest surviving member of B (0: all of them survive)
   if (n != 0) {
-    for (uint32_t i = tid; i < n; i += kSoloThreads) words[i] |= (uint64_t)(~(uint32_t)ci[ats[i]]);
+    if (!tie_mode)
+      for (uint32_t i = tid; i < n; i += kSoloThreads) words[i] |= (uint64_t)(~(uint32_t)ci[ats[i]]);
     __syncthreads();
     if (n <= kSoloRankDirect) {
       if (tid < n) {  // thread t counts the entries better than entry t: the need-th best is the cut
@@ -621,14 +693,14 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
 #pragma unroll
           for (int e = 0; e < 8; ++e) better += got[e] > mine ? 1u : 0u;
         }
-        if (better + 1 == f.need) cut_word = mine;
+        if (better + 1 == need) cut_word = mine;
       }
       __syncthreads();
       cut = cut_word;
     } else {  // a longer list: the block-wide radix select over its words (all distinct)
       auto key_at = [&](uint32_t i) -> uint64_t { return words[i]; };
       auto index_at = [&](uint32_t) -> uint64_t { return 0; };
-      cut = select::find_cut<uint64_t, 64>(sh, n, f.need, 1, key_at, index_at).T;
+      cut = select::find_cut<uint64_t, 64>(sh, n, need, 1, key_at, index_at).T;
     }
     for (uint32_t i = tid; i < n; i += kSoloThreads) before += (ats[i] < g * kSoloThreads && words[i] >= cut) ? 1u : 0u;
   }
