@@ -462,7 +462,7 @@ constexpr int kSoloWaves = kSoloThreads / select::kWave;
 constexpr uint32_t kSoloRankDirect = 512;
 static_assert((uint32_t)kSoloThreads == kSoloSegment, "a thread's u-th candidate lies in segment u");
 
-template <typename E, int NPT, bool OWN_RANGE, bool TIES = (sizeof(typename E::raw_t) == 1)>
+template <typename E, int NPT, bool OWN_RANGE, bool TIES = (sizeof(typename E::raw_t) == 1 || NPT <= 16)>
 __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t groups, int index_bits, const uint2* __restrict__ range, uint32_t entries,
@@ -649,7 +649,10 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     if (g != 0) return;
     auto key_at = [&](uint32_t i) -> key_t { return E::key(cv[i]); };
     auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)ci[i]; };
-    const select::Cut<key_t> whole = select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
+    // (the key of the k-th best is known by now, shift == 0: the digit is its offset from `low`;
+    // f.need of its candidates belong)
+    const select::Cut<key_t> whole =
+        select::cut_among_ties<key_t>(sh, k0, (key_t)(low + f.digit), f.need, index_bits, key_at, index_at);
     auto survives = [&](uint32_t i) -> bool {
       const key_t kk = key_at(i);
       if (kk != whole.T) return kk > whole.T;

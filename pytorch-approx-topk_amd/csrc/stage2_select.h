@@ -138,6 +138,26 @@ template <typename key_t> struct Cut {
   uint64_t index_cut;  // ~0: every tie survives
 };
 
+// The largest index taken among the candidates with key == T when `need` of them
+// (those with the lowest indices) belong to the result: radix passes over the
+// indices, least index first.  The histogram copies must be zero on entry.
+template <typename key_t, typename KeyAt, typename IndexAt, typename Sh>
+__device__ __forceinline__ uint64_t index_cut_among_ties(Sh& sh, uint32_t k0, key_t T, uint32_t need, int index_bits,
+                                                         KeyAt key_at, IndexAt index_at) {
+  uint64_t iprefix = 0, imask = 0;
+  for (int shift = ((index_bits + 7) / 8 - 1) * 8; shift >= 0; shift -= 8) {
+    radix_pass<false>(sh, k0, need, [&](uint32_t i) -> int {
+      if (key_at(i) != T) return -1;
+      const uint64_t idx = index_at(i);
+      return (idx & imask) == iprefix ? (int)((uint32_t)(idx >> shift) & 0xffu) : -1;
+    });
+    iprefix |= (uint64_t)sh.digit << shift;
+    imask |= (uint64_t)0xff << shift;
+    need = sh.need;
+  }
+  return iprefix;
+}
+
 // key_at(i): order key of candidate i; index_at(i): its original index (only
 // read for candidates tied at T, and only when the tie group is cut).
 template <typename key_t, int KEY_BITS, typename KeyAt, typename IndexAt, typename Sh>
@@ -176,20 +196,19 @@ __device__ __forceinline__ Cut<key_t> find_cut(Sh& sh, uint32_t k0, uint32_t k, 
     __syncthreads();
     cut.index_cut = sh.index_cut;
   } else if (need < ties) {
-    uint64_t iprefix = 0, imask = 0;
-    for (int shift = ((index_bits + 7) / 8 - 1) * 8; shift >= 0; shift -= 8) {
-      radix_pass<false>(sh, k0, need, [&](uint32_t i) -> int {
-        if (key_at(i) != cut.T) return -1;
-        const uint64_t idx = index_at(i);
-        return (idx & imask) == iprefix ? (int)((uint32_t)(idx >> shift) & 0xffu) : -1;
-      });
-      iprefix |= (uint64_t)sh.digit << shift;
-      imask |= (uint64_t)0xff << shift;
-      need = sh.need;
-    }
-    cut.index_cut = iprefix;
+    cut.index_cut = index_cut_among_ties(sh, k0, cut.T, need, index_bits, key_at, index_at);
   }
   return cut;
+}
+
+// The same when the key T of the k-th best is already known, with more
+// candidates of that key than belong to the result: `need` of them do, the ones
+// with the lowest indices.
+template <typename key_t, typename KeyAt, typename IndexAt, typename Sh>
+__device__ __forceinline__ Cut<key_t> cut_among_ties(Sh& sh, uint32_t k0, key_t T, uint32_t need, int index_bits,
+                                                     KeyAt key_at, IndexAt index_at) {
+  clear_copies(sh);
+  return Cut<key_t>{T, index_cut_among_ties(sh, k0, T, need, index_bits, key_at, index_at)};
 }
 
 // Stable compaction: wave w owns a contiguous run of candidates.  fetch(i) is
