@@ -29,9 +29,10 @@
 // offsets, and so on, through the bits of the key and then of the index, until
 // the cut digit fits (every emit workgroup does this over the row's list in
 // global memory, which holds all of B; the one-launch form narrows over the key
-// bits and leaves a row with more than kListCap candidates of one key around
-// the cut to its first workgroup, with the block-wide radix select over all of
-// its candidates).  When stage 1 ends in kernels that can leave key ranges and the
+// bits of the keys in its registers and, in the forms built with TIES, over the
+// index bits; without TIES it leaves a row with more than kListCap candidates
+// of one key around the cut to its first workgroup, with radix passes over the
+// indices of all candidates of that key).  When stage 1 ends in kernels that can leave key ranges and the
 // histogram behind (KeyRangeOut: the streaming kernel's slabs and their merge),
 // the range and hist launches are skipped.  Results are those of the
 // one-workgroup kernel: same survivors, same order.
