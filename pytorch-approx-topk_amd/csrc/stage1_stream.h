@@ -732,6 +732,20 @@ __host__ __device__ constexpr int loads_in_flight(int dtype, int j, int vec, boo
   return (j <= 2 || (dtype == ATK_F32 && j >= kWideFromJ)) ? 8 : 4;
 }
 
+// Packed 16-bit queues of two or four entries over columns of at most
+// kShortColumn sub-rows, scanned by the general loop (run == 0: columns of 33-64
+// sub-rows), keep eight loads in flight instead of four: fp16 [256, 2^20]
+// k=65536 j=4 166 -> 149 us, [128, 2^20] k=32768 j=2 65.5 -> 60.5 us, [16, 2^22]
+// k=2^18 j=4 47.8 -> 45.3 us.  The exact short runs (columns of up to 32) gain
+// nothing from it, and with long columns eight lose (fp16 [1, 2^26] j=4 k_mult=2
+// 53.9 -> 62.1 us, [128, 2^20] k=16384 j=4 62.7 -> 74.8 us).
+constexpr uint32_t kShortColumn = 64;
+__host__ __device__ constexpr bool deep_loads_for_short_columns(int dtype, int j, int vec, bool packed, int run,
+                                                                uint32_t full_rows) {
+  return packed && elem_bytes(dtype) == 2 && vec == 8 && (j == 2 || j == 4) && run == 0 &&
+         full_rows <= kShortColumn;
+}
+
 template <typename E, int J, int V, bool PACKED, bool SHIFTED = false>
 using QueueFor = std::conditional_t<
     !PACKED,

@@ -14,6 +14,13 @@ static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typ
   if constexpr (PackedKey<E>::available) {
     if (pl.packed) {
       constexpr int UP = loads_in_flight(DtypeOf<E>::value, J, V, true);
+      if constexpr (deep_loads_for_short_columns(DtypeOf<E>::value, J, V, true, RUN, 0) && UP != 8) {
+        if (deep_loads_for_short_columns(DtypeOf<E>::value, J, V, true, RUN, g.full_rows)) {
+          hipLaunchKernelGGL((stream_kernel<E, J, V, W, 8, RUN, true>), grid, dim3(kWave * W), 0, stream, x, out, g,
+                             left);
+          return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+        }
+      }
       hipLaunchKernelGGL((stream_kernel<E, J, V, W, UP, RUN, true>), grid, dim3(kWave * W), 0, stream, x, out, g, left);
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }

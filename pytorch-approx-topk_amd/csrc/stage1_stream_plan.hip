@@ -148,7 +148,9 @@ bool describe_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_
                        ((uintptr_t)indices % 16 == 0) && (row_stride % vf == 0);
   const stream::Plan pl = stream::make_plan(rows, n, k0, j, layout, dtype, aligned);
   if (!pl.ok) return false;
-  const int loads = stream::loads_in_flight(dtype, j, pl.vec, pl.packed);
+  const int loads = stream::deep_loads_for_short_columns(dtype, j, pl.vec, pl.packed, pl.run, pl.full_rows)
+                        ? 8
+                        : stream::loads_in_flight(dtype, j, pl.vec, pl.packed);
   out += "stream_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) +
          ", V=" + std::to_string(pl.vec) + ", W=" + std::to_string(pl.waves) + ", U=" + std::to_string(loads) +
          ", RUN=" + std::to_string(pl.run) + ", PACKED=" + (pl.packed ? "1" : "0") + "> grid=" +

@@ -280,6 +280,18 @@ def test_fused_rows_shapes(n, k, j, k_mult):
     _check(cpu_randn((136, n), n + k), k, -1, j=j, k_mult=k_mult)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.int16])
+@pytest.mark.parametrize("rows,n,k,j", [(9, 49152, 2048, 2), (9, 49252, 4096, 4), (300, 32768, 2048, 4),
+                                        (5, 1 << 18, 16384, 4), (3, 33 * 2048 + 7, 4096, 2)])
+def test_packed_queues_over_columns_of_33_to_64_sub_rows(dtype, rows, n, k, j):
+    # 16-bit types, two or four entries per column, columns of 33-64 sub-rows: the general scan loop
+    # with eight loads in flight; ties, and a ragged last sub-row
+    g = torch.Generator().manual_seed(n + k + j)
+    x = torch.randint(-300, 300, (rows, n), generator=g)
+    x = (x / 8).to(dtype) if dtype.is_floating_point else x.to(dtype)
+    _check(x, k, -1, j=j)
+
+
 @pytest.mark.parametrize("dtype,rows,n,k,j,k_mult", [
     (torch.float16, 130, 65536, 4096, 4, 8),     # 32768 candidates: 128 KiB of LDS
     (torch.bfloat16, 9, 65536, 3072, 1, 8),      # 24576 candidates, few rows
