@@ -3,7 +3,8 @@
 
 Covers the grid of the reference's benchmarks/measure_speed.py:264-327
 (n in 2^12..2^16, batch in {128, 32}, k in {64, n/8}, fp32; torch.topk, the
-approximate top-k at j in {1, 2, 4}, and the torch-level bucketed arg-max), once
+approximate top-k at j in {1, 2, 4}, and the torch-level bucketed arg-max, the last two
+also under torch.compile as there, :66-71), once
 with plain launches and once with the inner loop captured in a HIP graph, timed
 with events as benchmarks/measure_speed.py:98-146 does, a device-side spin queued
 ahead of every timed repetition included (:141): the host gets ahead of the GPU
@@ -82,6 +83,13 @@ def time_calls(call: Callable[[int], Any], refresh: Callable[[], None], n_outer:
     return [start.elapsed_time(stop) / 1e3 / n_inner for start, stop in events]
 
 
+def compiled_method(fn: Callable) -> Callable:
+    """`fn` under torch.compile as the reference's sweep compiles its methods
+    (benchmarks/measure_speed.py:66-71): mode "default", one graph, static shapes."""
+    torch.compiler.reset()
+    return torch.compile(fn, mode="default", fullgraph=True, dynamic=False)
+
+
 # (batch, n, k, j, k_mult) of the reference's own recorded rows, fp16, and the method they timed
 REFERENCE_ROWS = (
     [("approx_topk.topk", 256, 1 << 20, k, j, 1) for k in (65536, 16384) for j in (1, 2, 4)]
@@ -130,16 +138,21 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default="measure_speed.jsonl")
     ap.add_argument("--quick", action="store_true", help="fewer repetitions")
+    ap.add_argument("--no-compile", action="store_true", help="leave out the torch.compile variants")
     ap.add_argument("--reference-rows", action="store_true",
                     help="the shapes of the reference's own recorded measurements (fp16) instead of the grid")
     args = ap.parse_args()
     if args.reference_rows:
         return reference_rows(args.out, args.quick)
 
-    methods: list[tuple[str, Callable, dict]] = [("torch.topk", exact_topk, {})]
-    for j in (1, 2, 4):
-        methods.append((f"approx_topk.topk j={j}", approx_topk, dict(j=j, k_mult=1)))
-    methods.append(("bucketed_argmax.topk_torch", bucketed_argmax.topk_torch, dict(interleaved=True)))
+    # (name, function, arguments, compiled): as the reference does (benchmarks/measure_speed.py:66-71,
+    # 292-296), the approximate top-k and the torch-level arg-max are also timed under
+    # torch.compile(mode="default", fullgraph=True, dynamic=False)
+    methods: list[tuple[str, Callable, dict, bool]] = [("torch.topk", exact_topk, {}, False)]
+    for compiled in (False, True):
+        for j in (1, 2, 4):
+            methods.append((f"approx_topk.topk j={j}", approx_topk, dict(j=j, k_mult=1), compiled))
+        methods.append(("bucketed_argmax.topk_torch", bucketed_argmax.topk_torch, dict(interleaved=True), compiled))
 
     modes = [dict(graph=False, n_outer=64 if args.quick else 512, n_inner=1),
              dict(graph=True, n_outer=4 if args.quick else 16, n_inner=128)]
@@ -149,15 +162,20 @@ def main() -> int:
             n = 2 ** exp
             xs = torch.zeros(mode["n_inner"], batch, n, device="cuda")
             for k in (64, n // 8):
-                for name, fn, kwargs in methods:
-                    durations = time_calls(lambda i: fn(xs[i], k=k, dim=1, **kwargs)[0],
+                for name, fn, kwargs, compiled in methods:
+                    if args.no_compile and compiled:
+                        continue
+                    method = compiled_method(fn) if compiled else fn
+                    durations = time_calls(lambda i: method(xs[i], k=k, dim=1, **kwargs)[0],
                                            lambda: xs.normal_(), **mode)
                     mean = sum(durations) / len(durations)
-                    row = dict(method=name, args=kwargs, batch_size=batch, topk_size=n, k=k, dtype="float32",
+                    row = dict(method=name, args=kwargs, compile="default" if compiled else None, batch_size=batch,
+                               topk_size=n, k=k, dtype="float32",
                                hip_graphs=mode["graph"], n_outer=mode["n_outer"], n_inner=mode["n_inner"],
                                duration=durations, input_GBps=4 * n * batch / mean / 1e9, device=device)
                     print(json.dumps(row), file=out, flush=True)
-                    print(f"n=2^{exp} batch={batch} k={k} graph={mode['graph']} {name}: "
+                    print(f"n=2^{exp} batch={batch} k={k} graph={mode['graph']} {name}"
+                          f"{' compiled' if compiled else ''}: "
                           f"{mean * 1e6:.1f} us, {row['input_GBps']:.0f} GB/s", flush=True)
     return 0
 

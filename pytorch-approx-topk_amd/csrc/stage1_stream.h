@@ -58,10 +58,19 @@ __host__ __device__ constexpr int full_vec(int elem_size) { return elem_size == 
 
 // LDS a workgroup of `waves` needs to hand the queues of waves 1.. to wave 0,
 // and the most the planner lets it use.
-__host__ __device__ constexpr size_t merge_lds_bytes(int vec, int j, int waves, int cmp_size) {
-  return (size_t)(waves - 1) * vec * j * kWave * (cmp_size + 4);
+// `entry_bytes`: a queue entry as handed over (the packed queues: one 32-bit word;
+// else the value in compare form and the sub-row number).
+__host__ __device__ constexpr size_t merge_lds_bytes(int vec, int j, int waves, int entry_bytes) {
+  return (size_t)(waves - 1) * vec * j * kWave * entry_bytes;
 }
 constexpr size_t kMergeLdsLimit = 48 * 1024;
+// Packed 16-bit queues may take more: eight waves of four entries over eight
+// columns a lane (56 KiB; two workgroups per CU, which is what their registers
+// allow anyway).
+constexpr size_t kMergeLdsLimitPacked = 56 * 1024;
+__host__ __device__ constexpr size_t merge_lds_limit(int entry_bytes) {
+  return entry_bytes == 4 ? kMergeLdsLimitPacked : kMergeLdsLimit;
+}
 
 // Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).
 template <typename F, int... I>
@@ -399,7 +408,8 @@ template <int J, int FILLED = J> __device__ __forceinline__ void insert_word(uin
   else col[J - 1] = col[J - 1] > word ? col[J - 1] : word;
 }
 
-template <typename E, int J, int V, bool SHIFTED = false> struct PackedQueue {
+// LEAN: the three-operation keys and the shorter first inserts (see keys2_lean).
+template <typename E, int J, int V, bool SHIFTED = false, bool LEAN = !SHIFTED> struct PackedQueue {
   using raw_t = typename E::raw_t;
   using K = PackedKey<E>;
   static_assert(sizeof(raw_t) == 2 && (V % 2 == 0 || V == 1), "packed queues hold 16-bit elements");
@@ -438,16 +448,15 @@ template <typename E, int J, int V, bool SHIFTED = false> struct PackedQueue {
   __device__ static __forceinline__ void insert(uint32_t (&col)[J], uint32_t word) { insert_word<J>(col, word); }
   template <int FILLED> __device__ __forceinline__ void take(const Pack<raw_t, V>& pk, uint32_t p) {
     const uint32_t pinv = low_half(p);
-    // the lean keys and the shorter first inserts: not in the one-kernel path (SHIFTED), see keys2_lean
-    constexpr int F = SHIFTED ? J : FILLED;
+    constexpr int F = LEAN ? FILLED : J;
     if constexpr (V == 1) {
-      const uint32_t keys = SHIFTED ? K::keys2(pk.e[0], screen) : K::keys2_lean(pk.e[0], screen);
+      const uint32_t keys = LEAN ? K::keys2_lean(pk.e[0], screen) : K::keys2(pk.e[0], screen);
       insert_word<J, F>(q[0], (keys << 16) | pinv);
     } else {
       ATK_STATIC_FOR(d, V / 2) {
         uint32_t x;  // elements 2d (low half) and 2d+1 (high half) as loaded
         __builtin_memcpy(&x, &pk.e[2 * d], 4);
-        const uint32_t keys = SHIFTED ? K::keys2(x, screen) : K::keys2_lean(x, screen);
+        const uint32_t keys = LEAN ? K::keys2_lean(x, screen) : K::keys2(x, screen);
         insert_word<J, F>(q[2 * d], (keys << 16) | pinv);
         insert_word<J, F>(q[2 * d + 1], (keys & 0xffff0000u) | pinv);
       } ATK_STATIC_END;
@@ -456,12 +465,12 @@ template <typename E, int J, int V, bool SHIFTED = false> struct PackedQueue {
   // one more element for column VI, when `valid` (the word 0 changes nothing)
   template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
     uint32_t scr = screen;
-    const uint32_t keys = SHIFTED ? K::keys2((uint32_t)raw, scr) : K::keys2_lean((uint32_t)raw, scr);  // the empty high half screens as +0
+    const uint32_t keys = LEAN ? K::keys2_lean((uint32_t)raw, scr) : K::keys2((uint32_t)raw, scr);  // the empty high half screens as +0
     if (valid) screen = scr;
     insert(q[VI], valid ? ((keys << 16) | low_half(p)) : 0u);
   }
   __device__ __forceinline__ bool poisoned() const {
-    if constexpr (SHIFTED) {
+    if constexpr (!LEAN) {
       return __ballot(K::special(screen)) != 0;
     } else {
       bool nan = K::special_lean(screen);
@@ -883,15 +892,75 @@ __device__ __forceinline__ void exact_columns(const typename E::raw_t* __restric
   }
 }
 
+// The rest of a wave's scan once its queues are full: sub-rows [p, p1) of this
+// lane's columns, `next` pointing at sub-row p, U loads in flight: an odd batch
+// of fewer than U, then batches of U that are refilled while they are consumed.
+// Loads and their uses are kept in the same basic block wherever a load is
+// outstanding across them, so that the wait counts are exact.
+template <typename E, int J, int V, int U, typename Queue>
+__device__ __forceinline__ void scan_rest(const typename E::raw_t* next, int64_t b, uint32_t p, uint32_t p1,
+                                          Queue& queue) {
+  using raw_t = typename E::raw_t;
+  auto load_next = [&]() __attribute__((always_inline)) {
+    const Pack<raw_t, V> pk = load_pack<raw_t, V>(next);
+    next += b;
+    return pk;
+  };
+  const uint32_t odd = (p1 - p) % U;
+  if (odd != 0) {  // fewer than U sub-rows, so that whole batches remain
+    Pack<raw_t, V> buf[U];
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u) {
+      if ((uint32_t)u < odd) buf[u] = load_next();
+    }
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u) {
+      if ((uint32_t)u < odd) queue.template take<J>(buf[u], p + u);
+    }
+    p += odd;
+  }
+  uint32_t batches = (p1 - p) / U;
+  if (batches != 0) {
+    Pack<raw_t, V> buf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) buf[u] = load_next();
+    for (; batches > 1; --batches) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const Pack<raw_t, V> cur = buf[u];
+        buf[u] = load_next();
+        queue.template take<J>(cur, p + u);
+      }
+      p += U;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) queue.template take<J>(buf[u], p + u);
+  }
+}
+
+// The row's partial sub-row: column c has one more element when c < rem (with a
+// padded row the other columns see the pad value there).  Its number is above
+// all others, so it comes last.
+template <typename E, int V, typename Queue>
+__device__ __forceinline__ void scan_partial_sub_row(const typename E::raw_t* __restrict__ xr, const Geom& g,
+                                                     int64_t col, bool live, Queue& queue) {
+  using raw_t = typename E::raw_t;
+  if (g.rem != 0) {
+    ATK_STATIC_FOR(v, V) {
+      const bool real = live && col + v < (int64_t)g.rem;
+      const raw_t* at = real ? xr + (int64_t)g.full_rows * g.b + col + v : xr;  // xr[0] always exists
+      const raw_t value = *at;
+      queue.template take_one<v>(real ? value : E::pad_raw, g.full_rows, real || (live && g.pad_tail != 0));
+    } ATK_STATIC_END;
+  }
+}
+
 // One wave's scan: folds sub-rows [p0, p1) (p1 - p0 >= J) of this lane's V
 // columns starting at `col` into `queue`, plus the row's partial sub-row when
 // `with_rem`.  `xr` is the row; lanes that are not `live` load column 0 and are
 // ignored by the caller.  RUN > 0 promises p1 - p0 == RUN (J <= RUN): all loads
 // are issued at once and the code is one straight line.  RUN == 0 takes any
-// length: the first J sub-rows, then an odd batch of fewer than U, then batches
-// of U that are refilled while they are consumed.  Loads and their uses are
-// kept in the same basic block wherever a load is outstanding across them, so
-// that the wait counts are exact.
+// length: the first J sub-rows, then the rest as scan_rest does.
 template <typename E, int J, int V, int U, int RUN, typename Queue>
 __device__ __forceinline__ void scan_run(const typename E::raw_t* __restrict__ xr, const Geom& g, int64_t col,
                                 bool live, uint32_t p0, uint32_t p1, bool with_rem, Queue& queue) {
@@ -912,55 +981,15 @@ __device__ __forceinline__ void scan_run(const typename E::raw_t* __restrict__ x
     for (int u = 0; u < RUN; ++u) buf[u] = load_next();
     ATK_STATIC_FOR(u, RUN) { queue.template take<(u < J ? u : J)>(buf[u], p0 + u); } ATK_STATIC_END;
   } else {
-    uint32_t p = p0;
     {  // the first J sub-rows fill the queues
       Pack<raw_t, V> buf[J];
 #pragma unroll
       for (int u = 0; u < J; ++u) buf[u] = load_next();
       ATK_STATIC_FOR(u, J) { queue.template take<u>(buf[u], p0 + u); } ATK_STATIC_END;
-      p += J;
     }
-    const uint32_t odd = (p1 - p) % U;
-    if (odd != 0) {  // fewer than U sub-rows, so that whole batches remain
-      Pack<raw_t, V> buf[U];
-#pragma unroll
-      for (int u = 0; u < U - 1; ++u) {
-        if ((uint32_t)u < odd) buf[u] = load_next();
-      }
-#pragma unroll
-      for (int u = 0; u < U - 1; ++u) {
-        if ((uint32_t)u < odd) queue.template take<J>(buf[u], p + u);
-      }
-      p += odd;
-    }
-    uint32_t batches = (p1 - p) / U;
-    if (batches != 0) {
-      Pack<raw_t, V> buf[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) buf[u] = load_next();
-      for (; batches > 1; --batches) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const Pack<raw_t, V> cur = buf[u];
-          buf[u] = load_next();
-          queue.template take<J>(cur, p + u);
-        }
-        p += U;
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) queue.template take<J>(buf[u], p + u);
-    }
+    scan_rest<E, J, V, U>(next, g.b, p0 + J, p1, queue);
   }
-  // the partial sub-row: column c has one more element when c < rem
-  // (with a padded row the other columns see the pad value there)
-  if (with_rem && g.rem != 0) {
-    ATK_STATIC_FOR(v, V) {
-      const bool real = live && col + v < (int64_t)g.rem;
-      const raw_t* at = real ? xr + (int64_t)g.full_rows * g.b + col + v : xr;  // xr[0] always exists
-      const raw_t value = *at;
-      queue.template take_one<v>(real ? value : E::pad_raw, g.full_rows, real || (live && g.pad_tail != 0));
-    } ATK_STATIC_END;
-  }
+  if (with_rem) scan_partial_sub_row<E, V>(xr, g, col, live, queue);
 }
 
 // The same scan for a wave that shares its column tile with `split` - 1 others

@@ -25,8 +25,14 @@ static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typ
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }
   }
-  hipLaunchKernelGGL((stream_kernel<E, J, V, W, U, RUN, false>), grid, dim3(kWave * W), 0, stream, x, out, g, left);
-  return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+  // (the general queues hand over twice the bytes of the packed ones: combinations of theirs
+  // beyond the LDS budget, which the planner never picks, are not compiled)
+  if constexpr (merge_lds_bytes(V, J, W, (int)sizeof(typename Cmp<E>::cmp_t) + 4) <= merge_lds_limit(8)) {
+    hipLaunchKernelGGL((stream_kernel<E, J, V, W, U, RUN, false>), grid, dim3(kWave * W), 0, stream, x, out, g, left);
+    return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+  } else {
+    return ATK_ERR_ARG;
+  }
 }
 
 template <typename E, int J, int V, int W>
@@ -36,7 +42,8 @@ static int launch_one(const Plan& pl, const typename E::raw_t* x, const Sink<typ
   if (groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
   const dim3 grid((unsigned)groups);
   // combinations the planner never picks are not compiled
-  if constexpr (merge_lds_bytes(V, J, W, sizeof(typename Cmp<E>::cmp_t)) <= kMergeLdsLimit) {
+  constexpr int kEntryBytes = PackedKey<E>::available ? 4 : (int)sizeof(typename Cmp<E>::cmp_t) + 4;
+  if constexpr (merge_lds_bytes(V, J, W, kEntryBytes) <= merge_lds_limit(kEntryBytes)) {
     if constexpr (V > 1) {  // exact short runs exist for the vector kernels only
       if (pl.run == 4) return launch_run<E, J, V, W, 4>(pl, x, out, g, grid, stream, left);
       if (pl.run == 8) return launch_run<E, J, V, W, 8>(pl, x, out, g, grid, stream, left);

@@ -18,6 +18,8 @@ constexpr int64_t kLongRun = 64;
 // hand-over costs more than the scan (measured at 16 sub-rows: 4 waves x 4 beat
 // 8 x 2 by 25-45 %).
 constexpr int64_t kMinRun = 4;
+// Fewest sub-rows per wave for which a workgroup may take more LDS than kMergeLdsLimit.
+constexpr int64_t kLongWaveRun = 16;
 // Buckets at least this long are folded when they do not fill a column tile
 // (measured down to 8: fp32 [32768, 1024] with 16 buckets 104 -> 22 us, bf16
 // 193 -> 32 us; [65536, 256] with 16 buckets 70 -> 31 us).
@@ -71,11 +73,16 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   // the HBM bandwidth: measured, 8 waves x 4 sub-rows beats 4 x 8 at the
   // headline shape), with every run at least max(j, 4) long and the LDS
   // hand-over within its budget.
-  const int cmp_size = es > 4 ? 8 : 4;
+  const int entry_bytes = pl.packed ? 4 : (es > 4 ? 8 : 4) + 4;
   int64_t cost[4] = {full, 0, 0, 0};
   int cands = 1;
   for (int cand = 2; cand <= 8; cand *= 2, ++cands) {
-    if (full / cand < (j > kMinRun ? j : kMinRun) || merge_lds_bytes(pl.vec, j, cand, cmp_size) > kMergeLdsLimit) break;
+    const size_t hand = merge_lds_bytes(pl.vec, j, cand, entry_bytes);
+    if (full / cand < (j > kMinRun ? j : kMinRun) || hand > merge_lds_limit(entry_bytes)) break;
+    // Beyond the usual budget (packed queues of four entries, eight waves: 56 KiB, two workgroups
+    // per CU) only for long runs.  Measured, fp16 [256, 2^20], j = 4: columns of 256 sub-rows
+    // 125 -> 117 us, [1, 2^26] k = 16384 k_mult = 2 63 -> 47 us, but columns of 64 (runs of 8) 150 -> 162 us.
+    if (hand > kMergeLdsLimit && full / cand < kLongWaveRun) break;
     cost[cands] = full / cand + (int64_t)(cand - 1) * j;
   }
   int64_t best = cost[0];

@@ -557,6 +557,10 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   // all 255) -- and their indices decide.  Built for the 1-byte types only: the code costs the
   // kernel 4-5 us whether it runs or not (it sits at its register limit).
   const bool tie_mode = TIES && cut_digit && f.count > kListCap;
+  // The list in LDS holds kListCap entries: a cut digit with more members (which, without
+  // TIES, no bits are left to narrow) is not listed at all; the row then goes to the
+  // whole-row path below.
+  const bool list_it = cut_digit && f.count <= kListCap;
   const uint32_t own = g * kSoloThreads + tid;  // this thread's candidate of segment g
   const bool own_valid = own < k0;
   // survivors above the cut digit (or in it, when it belongs whole) in the
@@ -573,7 +577,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     if ((uint32_t)u == g) own_key = key[u];
     if (ok && cut_digit && d == f.digit) {
       if constexpr (TIES) members |= 1u << u;
-      if (!tie_mode) {
+      if (list_it) {
         const uint32_t at = (uint32_t)u * kSoloThreads + tid;
         const uint32_t slot = atomicAdd(&list_count, 1u);
         words[slot] = (uint64_t)key[u] << 32;  // (the index follows below, for all members in one trip to memory)

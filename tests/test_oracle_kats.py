@@ -264,6 +264,40 @@ def test_argmax_matches_torch_max_on_padded_view():
         assert torch.equal(i, mi * k + torch.arange(k))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32, torch.float64, torch.uint8,
+                                   torch.int8, torch.int16, torch.int32, torch.int64])
+def test_argmax_pad_element_of_every_dtype(dtype):
+    # The padded positions hold the dtype's minimum (approx_topk/experimental/bucketed_argmax.py:22-31
+    # in the reference).  The torch-level restatement takes it from torch.finfo / torch.iinfo, the
+    # oracle from its own table of constants: they must agree where the pad shows -- in buckets
+    # that are all padding (k > n), and against rows that hold nothing but the minimum itself, where
+    # a pad one step too high would win a partly padded bucket.
+    import sys
+    import os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                                    "pytorch-approx-topk_amd"))
+    from approx_topk.experimental.bucketed_argmax import topk_torch
+
+    info = torch.finfo(dtype) if dtype.is_floating_point else torch.iinfo(dtype)
+    g = torch.Generator().manual_seed(11)
+    for n, k in [(10, 4), (23, 5), (7, 12), (3, 8), (64, 9)]:
+        if dtype.is_floating_point:
+            x = (torch.randn(4, n, generator=g) * 3).to(dtype)
+        else:
+            x = torch.randint(max(info.min, -50), min(info.max, 50) + 1, (4, n), generator=g).to(dtype)
+        x[1] = info.min                      # ties between the row's elements and the padding
+        x[2, ::2] = info.min
+        if dtype.is_floating_point:
+            x[3, 0] = float("-inf")          # below the pad: a bucket of -inf and padding yields the pad
+        for interleaved in (False, True):
+            want_v, want_i = topk_torch(x, k, 1, interleaved)
+            got_v, got_i = oracle.bucketed_argmax(x, k, 1, interleaved)
+            assert torch.equal(got_i, want_i), (dtype, n, k, interleaved)
+            # (compared as bit patterns through a same-width integer view)
+            view = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[x.element_size()]
+            assert torch.equal(got_v.view(view), want_v.view(view)), (dtype, n, k, interleaved)
+
+
 # ---- order key -------------------------------------------------------------
 
 def test_key_order_floats():

@@ -99,3 +99,44 @@ def test_noalloc_rejects_what_does_not_fit_and_bad_arguments():
     rc, _, _ = _call_noalloc(x, 1 << 20, 1, 1024)   # k0 > n
     assert rc == -3
     torch.cuda.synchronize()
+
+
+def test_noalloc_under_graph_capture_and_replay():
+    # The entry point is for callers that cannot allocate: captured into a HIP graph (after one
+    # eager call, which also looks up the scratch array's address) and replayed, with eager work
+    # in between, it gives the workspace version's result every time and allocates nothing.
+    g = torch.Generator().manual_seed(5)
+    rows, n, k0, j, k = 1, 1 << 22, 8192, 4, 4096                # slabs + merge + select over several workgroups
+    xs = [(torch.randint(-60, 61, (rows, n), generator=g).float() / 8).cuda() for _ in range(3)]
+    x = torch.empty_like(xs[0])
+    x.copy_(xs[0])
+    need, ev, ei = _call_with_workspace(x, k0, j, k)
+    assert 0 < need <= SCRATCH_BYTES
+    rc, v, i = _call_noalloc(x, k0, j, k)
+    torch.cuda.synchronize()
+    assert rc == 0 and _same(v, ev) and torch.equal(i, ei)
+
+    from approx_topk import _native
+    L = _native.lib()
+    values = torch.empty(rows, k, dtype=x.dtype, device="cuda")
+    indices = torch.empty(rows, k, dtype=torch.int64, device="cuda")
+    code = _native.dtype_code(x.dtype)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            before = torch.cuda.memory_stats()["allocation.all.allocated"]
+            rc = L.atk_topk_noalloc(x.data_ptr(), rows, n, x.stride(0), k0, j, k, 0, code, values.data_ptr(),
+                                    indices.data_ptr(), torch.cuda.current_stream().cuda_stream)
+            after = torch.cuda.memory_stats()["allocation.all.allocated"]
+        assert rc == 0
+        assert after == before                                   # nothing came from torch's allocator either
+    torch.cuda.current_stream().wait_stream(side)
+    for replay, src in enumerate(xs + xs[:1]):
+        x.copy_(src)
+        _, ev, ei = _call_with_workspace(x, k0, j, k)             # eager work between the replays
+        values.zero_(); indices.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _same(values, ev) and torch.equal(indices, ei), replay
