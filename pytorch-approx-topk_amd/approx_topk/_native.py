@@ -249,11 +249,16 @@ def topk(xs: torch.Tensor, k0: int, j: int, k: int, layout: int, index_dtype: to
     return values, indices
 
 
-def describe(xs: torch.Tensor, k0: int, j: int, k: int, layout: int = INTERLEAVED) -> str:
-    """The kernels a call on `xs` (top-k along the last dim) would launch, as text."""
+def describe(xs: torch.Tensor, k0: int, j: int, k: int, layout: int = INTERLEAVED,
+             values: torch.Tensor | None = None, indices: torch.Tensor | None = None) -> str:
+    """The kernels a call on `xs` (top-k along the last dim) would launch, as text.
+
+    The plan depends on the alignment of the output buffers as well: pass the ones the call
+    will write (slices of larger buffers may be misaligned); without them the outputs are taken
+    to be fresh `torch.empty` tensors, which are at least 256-byte aligned."""
     xs, rows, n, step = rows_view(xs)
     buf = ctypes.create_string_buffer(1024)
-    # outputs of torch.empty are at least 256-byte aligned: any such address stands for them
     check(lib().atk_describe(xs.data_ptr() if xs.numel() else 4096, rows, n, step, k0, j, k, layout,
-                             dtype_code(xs.dtype), 4096, 4096, buf, len(buf)))
+                             dtype_code(xs.dtype), values.data_ptr() if values is not None else 4096,
+                             indices.data_ptr() if indices is not None else 4096, buf, len(buf)))
     return buf.value.decode()

@@ -467,7 +467,7 @@ template <typename E, int NPT, bool OWN_RANGE, bool TIES = (sizeof(typename E::r
 __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t groups, int index_bits, const uint2* __restrict__ range, uint32_t entries,
-    typename E::raw_t* __restrict__ values, const IndexOut indices) {
+    typename E::raw_t* __restrict__ values, const IndexOut indices, uint32_t tie_lds) {
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
@@ -528,6 +528,28 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   // The cut digit holds more candidates than the list: they are counted again by
   // the next bits of their offsets, which narrows the digit, until its members
   // fit or no bits are left.
+  if (f.need != f.count && f.count > kListCap && shift != 0) {
+    // Members of one and the same key (a ReLU's zeros) are not told apart by any further level,
+    // and every level would add them up in one counter, a lane at a time (16384 of them: 20 us
+    // a level).  Found out first: some member leaves its key in LDS, and every thread compares
+    // its members with that one.  (`red` is free: the digit's place has been worked out.)
+    __syncthreads();
+    if (tid == 0) red[1] = 0;
+#pragma unroll
+    for (int u = 0; u < NPT; ++u)
+      if (valid(u) && ((key[u] - low) >> shift) == f.digit) red[0] = key[u];  // (any of them will do)
+    __syncthreads();
+    const uint32_t one = (uint32_t)__builtin_amdgcn_readfirstlane((int)red[0]);
+    bool other = false;
+#pragma unroll
+    for (int u = 0; u < NPT; ++u) other |= valid(u) && ((key[u] - low) >> shift) == f.digit && key[u] != one;
+    if (__ballot(other) != 0 && lane == 0) red[1] = 1;
+    __syncthreads();
+    if (red[1] == 0) {  // the digit is the key's offset from here on
+      f.digit = one - low;
+      shift = 0;
+    }
+  }
   while (f.need != f.count && f.count > kListCap && shift != 0) {
     const uint32_t finer = shift > (uint32_t)regs::kDigitBits ? shift - (uint32_t)regs::kDigitBits : 0u;
     const uint32_t mask = (1u << (shift - finer)) - 1u;
@@ -644,6 +666,85 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
         });
         if (need == count) floor_word = key_word | ((uint64_t)iprefix << ishift);
       }
+    }
+  }
+  if constexpr (!TIES) {
+    if (cut_digit && f.count > kListCap && tie_lds) {
+      // Thousands of candidates of one key around the cut (a ReLU's zeros), in the form that keeps
+      // 32 keys per thread and has no registers to spare for the index levels above: the inverted
+      // indices of all members (up to the whole row) are listed in LDS, which the launch sized for
+      // it, the block-wide radix select of stage2_select.h finds the need-th largest among them,
+      // and a second look at the members' indices counts the survivors of the segments before this
+      // one.  Every workgroup of the row does all of it.  (shift == 0: the digit is the key's offset.)
+      uint32_t* inv_list = reinterpret_cast<uint32_t*>(dyn_lds);
+      const uint32_t* ci_low = reinterpret_cast<const uint32_t*>(ci);  // (indices below 2^31: the planner's rule)
+      const uint32_t cut_key = low + f.digit;
+      // an index's inverted bits, moved to the top of the word: the select's digits start where
+      // the indices differ (their leading bits are all alike, and a histogram of one bin is slow)
+      const uint32_t up = 32u - (uint32_t)(index_bits < 32 ? index_bits : 32);
+      __syncthreads();  // the list's LDS may still be read as `words`
+      constexpr int kChunk = 8;
+#pragma unroll
+      for (int c0 = 0; c0 < NPT; c0 += kChunk) {
+        uint32_t iv[kChunk];
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+          const uint32_t i = (uint32_t)(c0 + e) * kSoloThreads + tid;
+          iv[e] = i < k0 ? ci_low[2u * i] : 0u;
+        }
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+          const bool member = valid(c0 + e) && key[c0 + e] == cut_key;
+          const uint64_t m = __ballot(member);
+          uint32_t base = 0;
+          if (lane == 0 && m != 0) base = atomicAdd(&list_count, (uint32_t)__popcll(m));
+          base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
+          if (member) inv_list[base + select::rank_in(m)] = ~iv[e] << up;
+        }
+      }
+      // the need-th largest of the listed words (distinct values: no ties among them), by levels
+      // of 11 bits over the list, from the top down to the last bit an index has
+      uint32_t cut_inv = 0, level = 32, left_need = f.need, left_count = f.count;
+      while (level > up) {
+        const uint32_t finer = level - up > (uint32_t)regs::kDigitBits ? level - (uint32_t)regs::kDigitBits : up;
+        const uint32_t mask = (1u << (level - finer)) - 1u;
+        __syncthreads();  // the list is complete; everyone has read `found`, wave 0 the histogram
+        for (uint32_t i = tid; i < (uint32_t)regs::kBins; i += kSoloThreads) hist[i] = 0;
+        __syncthreads();
+        for (uint32_t i = tid; i < f.count; i += kSoloThreads) {
+          const uint32_t v = inv_list[i];
+          if (level == 32u || (v >> level) == (cut_inv >> level)) atomicAdd(&hist[(v >> finer) & mask], 1u);
+        }
+        __syncthreads();
+        if (wave == 0) {
+          const regs::Found f2 = regs::find_bin_wave<false>(hist, left_need, left_count, lane);
+          if (lane == 0) found = f2;
+        }
+        __syncthreads();
+        const regs::Found f2 = found;
+        cut_inv |= f2.digit << finer;
+        left_need = f2.need;
+        left_count = f2.count;
+        level = finer;
+      }
+      // members that survive in the segments before this one
+#pragma unroll
+      for (int c0 = 0; c0 < NPT; c0 += kChunk) {
+        uint32_t iv[kChunk];
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+          const uint32_t i = (uint32_t)(c0 + e) * kSoloThreads + tid;
+          iv[e] = i < k0 ? ci_low[2u * i] : 0u;
+        }
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+          if ((uint32_t)(c0 + e) < g && valid(c0 + e) && key[c0 + e] == cut_key && (~iv[e] << up) >= cut_inv) ++before;
+        }
+      }
+      need = count;  // settled: the members at or above the floor survive, nothing is listed
+      floor_word = ((uint64_t)cut_key << 32) | (uint64_t)((cut_inv >> up) | ~(0xffffffffu >> up));
+      __syncthreads();  // the list's LDS goes back to `words` (the padding entries below)
+      if (tid == 0) list_count = 0;
     }
   }
   if (need != count && count > kListCap) {
@@ -811,20 +912,36 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
     const bool own_ranges = entries == 0 && !pl.solo;  // stage 1 left no key ranges
     if (own_ranges) entries = pl.groups;
     if (pl.solo) {
-      const size_t solo_lds = (size_t)(kListCap + 8) * (sizeof(uint64_t) + sizeof(uint32_t));
+      size_t solo_lds = (size_t)(kListCap + 8) * (sizeof(uint64_t) + sizeof(uint32_t));
+      // The form with 32 keys per thread of a 2- or 4-byte type lists the inverted indices of a
+      // tied row's members in LDS: room for the whole row (up to 128 KiB; one workgroup per CU
+      // is all that runs of this kernel anyway).
+      uint32_t tie_lds = 0;
+      if (sizeof(raw_t) > 1 && k0 > 16 * kSoloThreads) {
+        const size_t tie_bytes = (size_t)k0 * sizeof(uint32_t);
+        if (solo_lds < tie_bytes) solo_lds = tie_bytes;
+        tie_lds = 1;
+      }
       const dim3 solo_block(kSoloThreads);
       raw_t* out = static_cast<raw_t*>(values);
 #define ATK_SOLO(NPT, OWN)                                                                                       \
-  hipLaunchKernelGGL((chain_solo_kernel<E, NPT, OWN>), grid, solo_block, solo_lds, stream, cv, cand_indices,     \
-                     (uint32_t)k0, (uint32_t)k, pl.groups, index_bits, (const uint2*)range, entries, out, indices)
+  {                                                                                                              \
+    auto kern = chain_solo_kernel<E, NPT, OWN>;                                                                  \
+    if (solo_lds > 48 * 1024 &&                                                                                  \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,     \
+                            (int)solo_lds) != hipSuccess)                                                        \
+      return ATK_ERR_LAUNCH;                                                                                     \
+    hipLaunchKernelGGL(kern, grid, solo_block, solo_lds, stream, cv, cand_indices, (uint32_t)k0, (uint32_t)k,    \
+                       pl.groups, index_bits, (const uint2*)range, entries, out, indices, tie_lds);              \
+  }
       if (entries != 0) {
-        if (k0 <= 8 * kSoloThreads) ATK_SOLO(8, false);
-        else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16, false);
-        else ATK_SOLO(32, false);
+        if (k0 <= 8 * kSoloThreads) ATK_SOLO(8, false)
+        else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16, false)
+        else ATK_SOLO(32, false)
       } else {
-        if (k0 <= 8 * kSoloThreads) ATK_SOLO(8, true);
-        else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16, true);
-        else ATK_SOLO(32, true);
+        if (k0 <= 8 * kSoloThreads) ATK_SOLO(8, true)
+        else if (k0 <= 16 * kSoloThreads) ATK_SOLO(16, true)
+        else ATK_SOLO(32, true)
       }
 #undef ATK_SOLO
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;

@@ -182,6 +182,32 @@ def test_chain_select_of_identical_candidates(k0):
     assert torch.equal(v[1].cpu(), torch.cat([torch.full((k0 // 2,), 5.0), torch.full((1234,), 2.0)]))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.int32])
+@pytest.mark.parametrize("rows,k0,zeros,k", [
+    (1, 32768, 16384, 24576),    # a ReLU's zeros: the cut takes half of 16384 equal keys
+    (3, 32768, 9000, 27000),     # ... of 9000, several rows
+    (2, 20000, 12000, 13000),    # a row that does not fill its last segment
+    (1, 32768, 32768, 5),        # nothing but the one key
+    (1, 30000, 8192, 21808 + 1), # one zero survives: the lowest index of all
+])
+def test_one_launch_select_of_rows_with_thousands_of_one_key_at_the_cut(dtype, rows, k0, zeros, k):
+    # 16385-32768 candidates of a 2- or 4-byte type: the one-launch form with 32 keys per thread, whose
+    # tied rows list the members' indices in LDS; every workgroup of the row must come to the same cut
+    g = torch.Generator().manual_seed(k0 + zeros)
+    if dtype.is_floating_point:
+        cv = torch.rand(rows, k0, generator=g) + 0.5
+    else:
+        cv = torch.randint(1, 30000, (rows, k0), generator=g)
+    for r in range(rows):
+        cv[r, torch.randperm(k0, generator=g)[:zeros]] = 0
+    cv = cv.to(dtype)
+    bound = 1 << 22
+    ci = torch.stack([torch.randperm(bound, generator=g)[:k0] for _ in range(rows)])
+    v, i = _select(cv, ci, k, bound)
+    ev, ei = oracle.stage2(cv, ci, k)
+    assert_same(v, i, ev, ei, f"{dtype} rows={rows} k0={k0} zeros={zeros} k={k}")
+
+
 def test_chain_select_needs_no_cut_when_the_digit_belongs_whole():
     # k falls exactly on a boundary between two values: every member of the cut digit survives
     k0 = 16384
