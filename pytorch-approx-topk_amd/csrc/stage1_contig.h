@@ -58,6 +58,8 @@ struct Geom {
   uint32_t groups;       // workgroups per row
   uint32_t slabs;        // > 1 (only with chunks > 1): workgroups sharing a bucket's chunks
   uint32_t slab_chunks;  // least chunks per slab: slab s takes chunks [s * chunks / slabs, (s + 1) * chunks / slabs)
+  uint32_t fast;         // the shape allows scan_even (see there)
+  uint32_t wide_out;     // the outputs allow 16-byte stores (filled in at launch)
 };
 
 // How a thread's queue holds values: in compare form (fast; no NaN may be
@@ -247,6 +249,149 @@ __device__ __forceinline__ bool scan_buckets(const typename E::raw_t* __restrict
   return true;
 }
 
+// LDS placement of scan_even: the span as the packs it was loaded in, 16 bytes of
+// padding per 128, so that the 16-byte reads of threads whose pieces lie a multiple of 32
+// words apart fall on different banks.
+// (`pack_bytes`: 16, or 8 for the 1-byte types, which load eight elements at a time)
+__host__ __device__ constexpr uint32_t even_offset(uint32_t pack, uint32_t pack_bytes) {
+  return pack * pack_bytes + ((pack * pack_bytes) >> 7) * 16u;
+}
+
+// The same pass for the shapes that allow it, with the register queues of the
+// streaming kernel (stage1_stream.h: one 32-bit word per entry for 8- and 16-bit
+// types, one 64-bit word for fp32 with J >= 2; about half the instructions per
+// element of the general form) and 16-byte LDS accesses: buckets of one length
+// (no remainder), whole within the span (no chunks), 16-byte loads from the
+// row, element types of at most four bytes, and pieces that are whole 16-byte
+// packs, so that every thread reads aligned packs only.  Positions are kept
+// relative to the bucket (packed entries hold 16 or 24 bits of them).  Returns
+// false, having written nothing, when a NaN was met (the caller then runs the
+// exact pass).
+template <typename E, int J, int V, bool PACKED>
+__device__ __forceinline__ bool scan_even(const typename E::raw_t* __restrict__ xr,
+                                          typename E::raw_t* __restrict__ values, const IndexOut& indices,
+                                          int64_t row, uint32_t group, const Geom& g, unsigned char* lds) {
+  using raw_t = typename E::raw_t;
+  using M = MergeWord<E>;
+  using word_t = typename M::word_t;
+  using Queue = stream::QueueFor<E, J, 1, PACKED>;
+  constexpr int N = J == 3 ? 4 : J;
+  constexpr uint32_t kPer = V;                                   // elements of a pack
+  constexpr uint32_t kPackBytes = V * (uint32_t)sizeof(raw_t);   // 16, or 8 for the 1-byte types
+  static_assert(V > 1 && sizeof(raw_t) <= 4 && V >= J, "whole packs, queues filled by the first");
+
+  const uint32_t t = threadIdx.x;
+  const uint32_t pieces = 1u << g.pieces_log2;
+  const uint32_t per_group = kThreads >> g.pieces_log2;  // buckets per workgroup
+  const uint32_t c0 = group * per_group;
+  const uint32_t c = c0 + (t >> g.pieces_log2);
+  const uint32_t piece = t & (pieces - 1);
+  const bool has = c < g.b;
+  const uint32_t c1 = c0 + per_group < g.b ? c0 + per_group : g.b;
+  const uint32_t e0 = c0 * g.m, e1 = c1 * g.m;  // the span (e0 is a multiple of a pack)
+
+  // the span into LDS, a pack per thread and trip, kLoads loads in flight
+  const uint32_t packs = (e1 - e0) / kPer;
+  const int64_t inside = (g.n - (int64_t)e0) / kPer;
+  const uint32_t whole = inside <= 0 ? 0u : (inside < (int64_t)packs ? (uint32_t)inside : packs);
+  for (uint32_t base = 0; base < whole; base += kThreads * kLoads) {
+    Pack<raw_t, V> got[kLoads];
+    ATK_STATIC_FOR(u, kLoads) {
+      const uint32_t pk = base + u * kThreads + t;
+      got[u] = stream::load_pack<raw_t, V>(xr + e0 + (size_t)(pk < whole ? pk : whole - 1) * V);
+    } ATK_STATIC_END;
+    ATK_STATIC_FOR(u, kLoads) {
+      const uint32_t pk = base + u * kThreads + t;
+      if (pk < whole) *reinterpret_cast<Pack<raw_t, V>*>(lds + even_offset(pk, kPackBytes)) = got[u];
+    } ATK_STATIC_END;
+  }
+  for (uint32_t pk = whole + t; pk < packs; pk += kThreads) {  // packs that reach past the row's end
+    const uint32_t at = e0 + pk * V;
+    Pack<raw_t, V> got;
+    ATK_STATIC_FOR(e, V) { got.e[e] = (int64_t)at + e < g.n ? xr[at + e] : E::pad_raw; } ATK_STATIC_END;
+    *reinterpret_cast<Pack<raw_t, V>*>(lds + even_offset(pk, kPackBytes)) = got;
+  }
+  __syncthreads();
+
+  // this thread's piece: `count` elements from position `first` of its bucket on
+  const uint32_t count = g.m >> g.pieces_log2;
+  const uint32_t first = piece * count;
+  const uint32_t pack0 = ((c - c0) * g.m + first) / kPer;
+  Queue queue;
+  queue.reset();
+  if (has) {
+    auto pack_at = [&](uint32_t i) __attribute__((always_inline)) {
+      return *reinterpret_cast<const Pack<raw_t, V>*>(lds + even_offset(pack0 + i, kPackBytes));
+    };
+    Pack<raw_t, V> cur = pack_at(0);
+    ATK_STATIC_FOR(e, V) {
+      queue.template take<(e < J ? e : J)>(Pack<raw_t, 1>{{cur.e[e]}}, first + e);
+    } ATK_STATIC_END;
+    const uint32_t trips = count / kPer;
+    for (uint32_t i = 1; i < trips; ++i) {
+      cur = pack_at(i);
+      ATK_STATIC_FOR(e, V) { queue.template take<J>(Pack<raw_t, 1>{{cur.e[e]}}, first + i * kPer + e); } ATK_STATIC_END;
+    }
+  }
+  if (__syncthreads_or(queue.poisoned())) return false;  // (also: the span is no longer read)
+
+  // combine the pieces of every bucket
+  const uint32_t start = c * g.m;
+  word_t acc[N], in[N];
+  ATK_STATIC_FOR(sl, N) { acc[sl] = M::empty(); in[sl] = M::empty(); } ATK_STATIC_END;
+  if (has) {
+    ATK_STATIC_FOR(sl, J) {
+      acc[N - J + sl] = M::from_key(queue.template key<0, sl>(), start + queue.template position<0, sl>());
+    } ATK_STATIC_END;
+  }
+  if (pieces > 1) {
+    word_t* lists = reinterpret_cast<word_t*>(lds);  // [N][kThreads]
+    for (uint32_t half = pieces / 2; half >= 1; half /= 2) {
+      if (piece >= half && piece < 2 * half) {
+        ATK_STATIC_FOR(sl, N) { lists[sl * kThreads + t] = acc[sl]; } ATK_STATIC_END;
+      }
+      __syncthreads();
+      if (piece < half) {
+        ATK_STATIC_FOR(sl, N) { in[sl] = lists[sl * kThreads + t + half]; } ATK_STATIC_END;
+        stream::merge_best<M, N>(acc, in);
+      }
+    }
+  }
+  if (has && piece == 0) {
+    const int64_t o = (row * g.b + c) * J;
+    if constexpr (J == 2 || J == 4) {
+      if (g.wide_out != 0) {  // a bucket's entries in one store of values and 16-byte stores of indices
+        Pack<raw_t, J> pv;
+        uint32_t p[J];
+        ATK_STATIC_FOR(sl, J) {
+          p[sl] = M::pos(acc[N - J + sl]);
+          pv.e[sl] = (int64_t)p[sl] < g.n ? stream::element_of<E>(acc[N - J + sl], xr, p[sl]) : E::pad_raw;
+        } ATK_STATIC_END;
+        if (values != nullptr) *reinterpret_cast<Pack<raw_t, J>*>(values + o) = pv;
+        if (indices.narrow) {
+          Pack<int32_t, J> pi;
+          ATK_STATIC_FOR(sl, J) { pi.e[sl] = (int32_t)p[sl]; } ATK_STATIC_END;
+          *reinterpret_cast<Pack<int32_t, J>*>(static_cast<int32_t*>(indices.base) + o) = pi;
+        } else {
+          ATK_STATIC_FOR(h, J / 2) {
+            Pack<int64_t, 2> pi;
+            pi.e[0] = (int64_t)p[2 * h];
+            pi.e[1] = (int64_t)p[2 * h + 1];
+            reinterpret_cast<Pack<int64_t, 2>*>(static_cast<int64_t*>(indices.base) + o)[h] = pi;
+          } ATK_STATIC_END;
+        }
+        return true;
+      }
+    }
+    ATK_STATIC_FOR(sl, J) {
+      const uint32_t p = M::pos(acc[N - J + sl]);
+      if (values != nullptr) values[o + sl] = (int64_t)p < g.n ? stream::element_of<E>(acc[N - J + sl], xr, p) : E::pad_raw;
+      indices.put(o + sl, p);
+    } ATK_STATIC_END;
+  }
+  return true;
+}
+
 // E: element traits; J: entries kept per bucket; V: elements per load (16
 // bytes' worth when the row allows it, else 1).
 template <typename E, int J, int V>
@@ -259,6 +404,19 @@ __global__ __launch_bounds__(kThreads) void contig_kernel(const typename E::raw_
   const uint32_t group = blockIdx.x - row32 * g.groups;
   const int64_t row = row32;
   const typename E::raw_t* xr = x + row * g.row_stride;
+  bool done = false;
+  if constexpr (V > 1 && sizeof(typename E::raw_t) <= 4) {
+    if (g.fast != 0) {
+      constexpr bool kPackable = stream::PackedKey<E>::available;
+      done = scan_even<E, J, V, kPackable>(xr, values, indices, row, group, g, contig_lds);
+      if (done) return;
+      if constexpr (Cmp<E>::has_nan) {
+        __syncthreads();
+        scan_buckets<E, J, V, KeyForm<E>>(xr, values, indices, partial, row, group, g, contig_lds);
+      }
+      return;
+    }
+  }
   if (scan_buckets<E, J, V, CmpForm<E>>(xr, values, indices, partial, row, group, g, contig_lds)) return;
   if constexpr (Cmp<E>::has_nan) {
     __syncthreads();

@@ -34,6 +34,7 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
   using raw_t = typename E::raw_t;
   Geom g = pl.geom;
   g.row_stride = row_stride;
+  g.wide_out = ((uintptr_t)values % 16 == 0 && (uintptr_t)indices.base % 16 == 0) ? 1u : 0u;
   const raw_t* xs = static_cast<const raw_t*>(x);
   raw_t* vs = static_cast<raw_t*>(values);
   switch (j) {

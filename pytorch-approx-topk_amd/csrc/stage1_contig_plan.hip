@@ -69,6 +69,19 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
   const size_t data_bytes = (size_t)(span + ((span >> 5) + 1) * pad_elems(es)) * es;
   const size_t list_bytes = (size_t)4 * kThreads * (es == 8 ? 16 : 8);
   pl.lds_bytes = ((data_bytes > list_bytes ? data_bytes : list_bytes) + 15) / 16 * 16;
+  // scan_even: buckets of one length, whole in the span, pieces of whole 16-byte packs, sub-row
+  // numbers that fit the packed entries
+  const int64_t per_pack = pl.vec;  // elements of a pack
+  g.fast = 0;
+  if (pl.vec > 1 && es <= 4 && r == 0 && g.chunks == 1 && (m >> lg) << lg == m && (m >> lg) % per_pack == 0 &&
+      (m >> lg) >= per_pack && per_pack >= j && (es != 2 || m <= (int64_t)stream::kPackedMaxSubRow)) {
+    const size_t packs = (size_t)(per_group * m) / per_pack;
+    const size_t even_bytes = even_offset((uint32_t)packs, (uint32_t)(per_pack * es)) + 16;
+    if (even_bytes <= 64 * 1024) {
+      g.fast = 1;
+      if (pl.lds_bytes < even_bytes) pl.lds_bytes = (even_bytes + 15) / 16 * 16;
+    }
+  }
   if (pl.lds_bytes > 64 * 1024) return pl;
   pl.ok = true;
   return pl;
@@ -94,7 +107,8 @@ bool describe_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_
   if (!pl.ok) return false;
   out += "contig_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + ", V=" +
          std::to_string(pl.vec) + "> grid=" + std::to_string(rows * (int64_t)pl.geom.groups) + " block=256 chunks=" +
-         std::to_string(pl.geom.chunks) + " slabs=" + std::to_string(pl.geom.slabs);
+         std::to_string(pl.geom.chunks) + " slabs=" + std::to_string(pl.geom.slabs) +
+         (pl.geom.fast ? " even" : "");
   if (pl.geom.slabs > 1) out += " + contig_merge_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + ">";
   return true;
 }
