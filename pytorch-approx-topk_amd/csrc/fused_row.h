@@ -31,7 +31,9 @@ using stream::kWave;
 // A value the fast queues cannot order (NaN) was loaded somewhere in the row:
 // stage 1 again with exact order keys, one thread per column, into the
 // candidate arrays in LDS.  All threads of the workgroup call this.
-template <typename E, int J, typename skey_t, typename pos_t>
+// CONTIG: bucket c is the run of g.full_rows adjacent elements from c * g.full_rows
+// on (no partial sub-row), not column c of the [full_rows][b] matrix.
+template <typename E, int J, bool CONTIG, typename skey_t, typename pos_t>
 __device__ __forceinline__ void redo_exact_into_lds(const typename E::raw_t* __restrict__ xr, const Geom& g,
                                                     skey_t* cand_key, pos_t* cand_pos) {
   using raw_t = typename E::raw_t;
@@ -39,8 +41,9 @@ __device__ __forceinline__ void redo_exact_into_lds(const typename E::raw_t* __r
     raw_t qv[J];
     uint32_t qp[J];
     stream::clear_exact<E, J>(qv, qp);
-    for (uint32_t p = 0; p < g.full_rows; ++p) stream::push_exact<E, J>(qv, qp, xr[(int64_t)p * g.b + c], p);
-    if (g.rem != 0) {
+    for (uint32_t p = 0; p < g.full_rows; ++p)
+      stream::push_exact<E, J>(qv, qp, xr[CONTIG ? c * (int64_t)g.full_rows + p : (int64_t)p * g.b + c], p);
+    if (!CONTIG && g.rem != 0) {
       if (c < (int64_t)g.rem)
         stream::push_exact<E, J>(qv, qp, xr[(int64_t)g.full_rows * g.b + c], g.full_rows);
       else if (g.pad_tail)
@@ -54,7 +57,7 @@ __device__ __forceinline__ void redo_exact_into_lds(const typename E::raw_t* __r
 // Stage 2 over the candidates parked in LDS (exact order keys and sub-row
 // numbers, candidate c*J + s belonging to column c): the block-wide radix
 // select, then the survivors in candidate order.  Starts with a barrier.
-template <typename E, int J, typename skey_t, typename pos_t, typename Sh>
+template <typename E, int J, bool CONTIG, typename skey_t, typename pos_t, typename Sh>
 __device__ __forceinline__ void select_from_lds(Sh& sh, const typename E::raw_t* __restrict__ xr, const Geom& g,
                                                 const skey_t* cand_key, const pos_t* cand_pos, uint32_t k0,
                                                 uint32_t k, int index_bits, int64_t row,
@@ -62,7 +65,10 @@ __device__ __forceinline__ void select_from_lds(Sh& sh, const typename E::raw_t*
   using raw_t = typename E::raw_t;
   using key_t = typename E::key_t;
   auto key_at = [&](uint32_t i) -> key_t { return cand_key[i]; };
-  auto index_at = [&](uint32_t i) -> uint64_t { return (uint64_t)cand_pos[i] * (uint64_t)g.b + i / J; };
+  auto index_at = [&](uint32_t i) -> uint64_t {
+    if constexpr (CONTIG) return (uint64_t)(i / J) * g.full_rows + cand_pos[i];
+    return (uint64_t)cand_pos[i] * (uint64_t)g.b + i / J;
+  };
   const select::Cut<key_t> cut =
       select::find_cut<key_t, E::key_bits>(sh, k0, k, index_bits, key_at, index_at);
 
@@ -163,9 +169,9 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
     if (split > 1 && hand_off != 0) __syncthreads();  // the hand-over area is reused by the next round
   }
 
-  if (__syncthreads_or(any_nan)) redo_exact_into_lds<E, J>(xr, g, cand_key, cand_pos);
+  if (__syncthreads_or(any_nan)) redo_exact_into_lds<E, J, false>(xr, g, cand_key, cand_pos);
   // (the select's first pass starts with a barrier, which also publishes the candidates)
-  select_from_lds<E, J>(sh, xr, g, cand_key, cand_pos, k0, k, index_bits, row, values, indices);
+  select_from_lds<E, J, false>(sh, xr, g, cand_key, cand_pos, k0, k, index_bits, row, values, indices);
 }
 
 // ---------------------------------------------------------------------------
@@ -185,10 +191,78 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
 // ---------------------------------------------------------------------------
 namespace regs = select::regs;
 
+// Stage 1 of a row whose buckets are runs of `m` adjacent elements of 16 to 64
+// bytes each (contiguous layout, every bucket as long).  A lane takes V buckets
+// kWave apart, `first` the first of them, so that the lanes of a wave load from
+// adjacent buckets, and loads a bucket whole, 16 bytes at a time, before it
+// feeds it to the bucket's queue with the place within the bucket as the sub-row
+// number: the loads of a wave then cover a stretch of the row back to back.
+// (With the lane's buckets side by side, lanes 128-256 bytes apart, and with one
+// load per bucket at a time, so that the second 16 bytes of a cache line are
+// asked for long after the first, fp32 [1024, 32768] with 2048 buckets took
+// 72-75 us against 47 for the interleaved row.)  AHEAD: the next bucket is loaded
+// before this one is fed.
+template <typename E, int J, int V, bool PACKED, bool AHEAD, typename Queue>
+__device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __restrict__ xr, uint32_t m,
+                                                   int64_t first, Queue& queue) {
+  using raw_t = typename E::raw_t;
+  constexpr int EPL = 16 / (int)sizeof(raw_t);  // elements per load
+  constexpr int kMaxLoads = 4;                  // a bucket is at most 64 bytes
+  static_assert(EPL >= J && EPL % 2 == 0, "the first load of a bucket fills its queue");
+  using Load = stream::Pack<raw_t, EPL>;
+  const raw_t* next = xr + first * (int64_t)m;
+  const int64_t apart = (int64_t)kWave * m;
+  const uint32_t loads = __builtin_amdgcn_readfirstlane(m / EPL);
+  queue.reset();
+  auto load_bucket = [&](Load (&buf)[kMaxLoads]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int c = 0; c < kMaxLoads; ++c) {
+      if (c == 0 || (uint32_t)c < loads) buf[c] = stream::load_pack<raw_t, EPL>(next + c * EPL);
+    }
+    next += apart;
+  };
+  auto feed = [&](auto v_c, const Load (&buf)[kMaxLoads]) __attribute__((always_inline)) {
+    constexpr int v = decltype(v_c)::value;
+    ATK_STATIC_FOR(c, kMaxLoads) {
+      if (c == 0 || (uint32_t)c < loads) {
+        ATK_STATIC_FOR(d, EPL / 2) {
+          constexpr int kFilled = (c == 0 && 2 * d < J) ? 2 * d : J;
+          if constexpr (PACKED) {
+            uint32_t x;
+            __builtin_memcpy(&x, &buf[c].e[2 * d], 4);
+            queue.template take_two<v, kFilled>(x, c * EPL + 2 * d);
+          } else {
+            queue.template take_two<v, kFilled>(buf[c].e[2 * d], buf[c].e[2 * d + 1], c * EPL + 2 * d);
+          }
+        } ATK_STATIC_END;
+      }
+    } ATK_STATIC_END;
+  };
+  if constexpr (AHEAD) {
+    Load buf[2][kMaxLoads];
+    load_bucket(buf[0]);
+    ATK_STATIC_FOR(v, V) {
+      if constexpr (v + 1 < V) load_bucket(buf[(v + 1) % 2]);
+      feed(std::integral_constant<int, v>{}, buf[v % 2]);
+    } ATK_STATIC_END;
+  } else {
+    ATK_STATIC_FOR(v, V) {
+      Load buf[kMaxLoads];
+      load_bucket(buf);
+      feed(std::integral_constant<int, v>{}, buf);
+    } ATK_STATIC_END;
+  }
+}
+
 // Packed queues of up to 16 entries per lane are held to 64 vector registers
 // (eight waves per SIMD: four 8-wave workgroups per CU); what does not fit is
 // spilled where the pressure peaks, in the rarely taken LDS path.
-template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED>
+// CONTIG: the row's buckets are contiguous runs of g.full_rows elements of at
+// most 64 bytes (no remainder, whole tiles, one wave per tile).  The scan differs,
+// the way an index is put together, and which buckets a lane holds: V buckets
+// kWave apart (bucket_of), so that a wave's candidates in their order are those
+// of every lane's first bucket, then of every lane's second, ...
+template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED, bool CONTIG = false>
 __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80)))
 __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_regs_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
@@ -226,9 +300,13 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
   const uint32_t p0 = __builtin_amdgcn_readfirstlane((uint32_t)(((uint64_t)g.full_rows * part) / split));
   const uint32_t p1 = __builtin_amdgcn_readfirstlane((uint32_t)(((uint64_t)g.full_rows * (part + 1)) / split));
   const bool has_tile = tile < tiles;
-  const int64_t col = (int64_t)tile * kTileCols + lane * V;
+  const int64_t col = (int64_t)tile * kTileCols + (CONTIG ? lane : lane * V);
   const bool live = has_tile && col < g.b;
   const bool mine = live && part == 0;  // this lane ends up holding candidates
+  // the bucket (column) of the lane's v-th queue
+  auto bucket_of = [&](int v) __attribute__((always_inline)) -> int64_t {
+    return CONTIG ? col + (int64_t)v * kWave : col + v;
+  };
 
   Queue queue;
   // packed entries: sub-row numbers 0..full_rows at the top of the low half, so
@@ -236,35 +314,43 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
   queue.set_position_shift(sizeof(pos_t) == 2 ? (uint32_t)__builtin_clz(g.full_rows | 1u) - 16u : 0u);
   bool any_nan = false;
   if (has_tile) {
-    if (split > 1) stream::scan_windows<E, J, V, U>(xr, g, col, live, part, split, part == split - 1, queue);
+    if constexpr (CONTIG) scan_short_buckets<E, J, V, PACKED, !PACKED>(xr, g.full_rows, col, queue);
+    else if (split > 1) stream::scan_windows<E, J, V, U>(xr, g, col, live, part, split, part == split - 1, queue);
     else stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, true, queue);
     any_nan = queue.poisoned();
   }
-  if (split > 1) {
-    if (has_tile && part > 0)
-      queue.hand_over(hand + (size_t)(tile * (split - 1) + (part - 1)) * Queue::kHandBytes, lane);
-    __syncthreads();
-    if (has_tile && part == 0) {
-      for (uint32_t w = 0; w + 1 < split; ++w)
-        queue.fold_in_interleaved(hand + (size_t)(tile * (split - 1) + w) * Queue::kHandBytes, lane);
+  if constexpr (!CONTIG) {
+    if (split > 1) {
+      if (has_tile && part > 0)
+        queue.hand_over(hand + (size_t)(tile * (split - 1) + (part - 1)) * Queue::kHandBytes, lane);
+      __syncthreads();
+      if (has_tile && part == 0) {
+        for (uint32_t w = 0; w + 1 < split; ++w)
+          queue.fold_in_interleaved(hand + (size_t)(tile * (split - 1) + w) * Queue::kHandBytes, lane);
+      }
     }
+    // Both histograms start at zero.  Waves that shared a tile must first be done
+    // with the hand-over area, which may lie in the same place.
+    if (split > 1) __syncthreads();
   }
-  // Both histograms start at zero.  Waves that shared a tile must first be done
-  // with the hand-over area, which may lie in the same place.
-  if (split > 1) __syncthreads();
   for (uint32_t i = tid * 4; i < 2 * regs::kHistWords; i += nt * 4)
     *reinterpret_cast<uint4*>(&hist[i]) = make_uint4(0, 0, 0, 0);
   if (tid == 0) rs.list_count = 0;
   const bool nan_row = __syncthreads_or(any_nan);
 
   // (keys are taken from the queues where they are used rather than kept: registers)
+  // (Packed entries carry the sub-row number below the key, which is the order of the
+  // indices of equal keys in the interleaved layout only: sub-row first, then column.)
+  constexpr bool kKeyHalf = CONTIG && PACKED;
   auto key_of = [&](auto e_c) __attribute__((always_inline)) -> sel_t {
     constexpr int e = decltype(e_c)::value;
+    if constexpr (kKeyHalf) return queue.template sel_key<e / J, e % J>() & (sel_t)0xffff0000u;
     return queue.template sel_key<e / J, e % J>();
   };
   auto index_of = [&](auto e_c) __attribute__((always_inline)) -> idx_t {
     constexpr int e = decltype(e_c)::value;
-    return (idx_t)queue.template position<e / J, e % J>() * (idx_t)g.b + (idx_t)(col + e / J);
+    if constexpr (CONTIG) return (idx_t)bucket_of(e / J) * (idx_t)g.full_rows + (idx_t)queue.template position<e / J, e % J>();
+    return (idx_t)queue.template position<e / J, e % J>() * (idx_t)g.b + (idx_t)bucket_of(e / J);
   };
 
   // MSB-first radix passes over sel_key.  After a pass the candidates still in
@@ -279,7 +365,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
   enum { kByPrefix, kByList, kGiveUp } how = kGiveUp;
   if (!nan_row) {
     int shift = Queue::sel_bits;
-    const int shift_end = queue.sel_constant_bits();
+    const int shift_end = kKeyHalf ? 16 : queue.sel_constant_bits();
     for (uint32_t pass = 0;; ++pass) {
       if (need == count) { how = kByPrefix; break; }
       if (count <= regs::kListMax) { how = kByList; break; }
@@ -324,14 +410,14 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
     // kListMax candidates equal to the cut key under sel_key (cut by index).
     __syncthreads();
     if (nan_row) {
-      redo_exact_into_lds<E, J>(xr, g, cand_key, cand_pos);
+      redo_exact_into_lds<E, J, CONTIG>(xr, g, cand_key, cand_pos);
     } else if (mine) {
       ATK_STATIC_FOR(e, NC) {
-        cand_key[col * J + e] = (skey_t)queue.template key<e / J, e % J>();
-        cand_pos[col * J + e] = (pos_t)queue.template position<e / J, e % J>();
+        cand_key[bucket_of(e / J) * J + e % J] = (skey_t)queue.template key<e / J, e % J>();
+        cand_pos[bucket_of(e / J) * J + e % J] = (pos_t)queue.template position<e / J, e % J>();
       } ATK_STATIC_END;
     }
-    select_from_lds<E, J>(sh, xr, g, cand_key, cand_pos, k0, k, index_bits, row, values, indices);
+    select_from_lds<E, J, CONTIG>(sh, xr, g, cand_key, cand_pos, k0, k, index_bits, row, values, indices);
     return;
   }
 
@@ -407,12 +493,27 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
     if (key == cut_key) s = index_of(std::integral_constant<int, e>{}) < cut_below;
     selected |= (mine && s) ? (1u << e) : 0u;
   } ATK_STATIC_END;
-  const uint32_t kept = (uint32_t)__popc(selected);
-  const uint32_t incl = regs::wave_scan(kept);
-  if (lane == kWave - 1) rs.wave_total[wave] = incl;
+  // Output slots follow the candidates' order: wave by wave, and within a wave lane by
+  // lane with the lane's candidates in a row, or (CONTIG) the lanes' v-th buckets
+  // together for one v after the other.  slot[r]: where the next survivor of run r goes.
+  constexpr int kRuns = CONTIG ? V : 1, kRunLen = NC / kRuns;
+  uint32_t slot[kRuns];
+  {
+    uint32_t before = 0;  // survivors of this wave in the runs so far
+    ATK_STATIC_FOR(r, kRuns) {
+      const uint32_t kept = (uint32_t)__popc((selected >> (r * kRunLen)) & (uint32_t)((1ull << kRunLen) - 1ull));
+      const uint32_t incl = regs::wave_scan(kept);
+      slot[r] = before + incl - kept;
+      before += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+    } ATK_STATIC_END;
+    if (lane == kWave - 1) rs.wave_total[wave] = before;
+  }
   __syncthreads();
-  uint32_t o = incl - kept;
-  for (uint32_t w = 0; w < wave; ++w) o += rs.wave_total[w];
+  {
+    uint32_t waves_before = 0;
+    for (uint32_t w = 0; w < wave; ++w) waves_before += rs.wave_total[w];
+    ATK_STATIC_FOR(r, kRuns) { slot[r] += waves_before; } ATK_STATIC_END;
+  }
   raw_t* ov = values + row * (int64_t)k;
   const int64_t oi = row * (int64_t)k;
   if constexpr (sizeof(idx_t) == 4 && sizeof(raw_t) <= 4) {
@@ -425,13 +526,14 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
       // (the barrier above).
       uint2* stage = reinterpret_cast<uint2*>(dyn_lds);
       ATK_STATIC_FOR(e, NC) {
-        if ((selected >> e) & 1u) stage[o] = queue.template staged<e / J, e % J>((uint32_t)col + e / J);
+        uint32_t& o = slot[e / kRunLen];
+        if ((selected >> e) & 1u) stage[o] = queue.template staged<e / J, e % J>((uint32_t)bucket_of(e / J));
         o += (selected >> e) & 1u;
       } ATK_STATIC_END;
       __syncthreads();
       auto result = [&](uint2 w, raw_t& value) __attribute__((always_inline)) -> uint32_t {
         const typename Queue::Unstaged u = queue.unstage(w);
-        const uint32_t index = u.sub_row * (uint32_t)g.b + u.column;
+        const uint32_t index = CONTIG ? u.column * g.full_rows + u.sub_row : u.sub_row * (uint32_t)g.b + u.column;
         value = u.raw;
         if (u.reread) value = xr[index];  // a zero: its sign is in the row
         return index;
@@ -472,8 +574,12 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_r
       return;
     }
   }
-  if (mine) queue.fix_zeros(xr, g.b, col);
+  if (mine) {
+    if constexpr (CONTIG) queue.fix_zeros(xr, 1, col * (int64_t)g.full_rows, (int64_t)kWave * g.full_rows);
+    else queue.fix_zeros(xr, g.b, col);
+  }
   ATK_STATIC_FOR(e, NC) {
+    uint32_t& o = slot[e / kRunLen];
     if ((selected >> e) & 1u) {
       if (o < k) {
         if (values != nullptr) ov[o] = queue.template raw<e / J, e % J>();
@@ -499,6 +605,7 @@ struct Plan {
   int index_bits;
   uint32_t hand_off;    // byte offset of the hand-over area in dynamic LDS (0: on top of the candidates)
   size_t lds_bytes;     // dynamic LDS
+  bool contig;          // contiguous buckets of a few elements each (in_registers only)
   bool in_registers;    // all tiles are scanned at once: the candidates stay in registers through stage 2
   bool staged;          // in_registers: the survivors are gathered in LDS and leave in whole-wave stores
 };

@@ -13,6 +13,13 @@ static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t row
     if (pl.in_registers) return ATK_ERR_ARG;  // (the register kernel is built for eight waves)
   } else if (pl.in_registers) {
     auto kern = fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED>;
+    // contiguous short buckets: 16-bit positions, elements of two (packed queues) or four bytes
+    constexpr int ES = (int)sizeof(typename E::raw_t);
+    if constexpr (sizeof(pos_t) == 2 && ((ES == 2 && PACKED) || ES == 4) && V == 4) {
+      if (pl.contig) kern = fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED, true>;
+    } else if (pl.contig) {
+      return ATK_ERR_ARG;  // the planner never asks for it
+    }
     if (pl.lds_bytes > 48 * 1024) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)pl.lds_bytes) != hipSuccess)

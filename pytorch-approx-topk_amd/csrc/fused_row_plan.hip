@@ -32,9 +32,49 @@ constexpr int64_t kManyRows = 1024, kAllCus = 256;
 constexpr size_t kShortRow = 128 * 1024, kLongRow = 512 * 1024;
 }  // namespace
 
+// Contiguous buckets, all of one length of 16 to 64 bytes (a quarter to a
+// sixteenth of the row's elements become candidates), elements of two or four
+// bytes: a lane of the register kernel loads its four buckets whole.  The
+// alternative is a stage-1 kernel that copies spans of buckets through LDS and
+// parks the candidates in HBM for a stand-alone select: fp16 [1024, 32768]
+// k=2048 j=4 k_mult=4 68.6 us that way.
+static Plan plan_short_buckets(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int dtype, bool aligned) {
+  Plan pl{};
+  pl.ok = false;
+  if (!aligned || rows > 0x7fffffffll) return pl;
+  if (k0 <= 0 || k <= 0 || k >= k0 || j < 1 || j > 4 || k0 % j) return pl;
+  const int es = elem_bytes(dtype);
+  if (es != 2 && es != 4) return pl;
+  if (rows < kMinRows && (size_t)n * es > kSoloRow) return pl;
+  const int64_t b = k0 / j;
+  if (n % b) return pl;
+  const int64_t m = n / b;
+  if ((m * es) % 16 || m * es > 64 || m < j) return pl;
+  pl.full_rows = (uint32_t)m;
+  pl.pos16 = true;
+  pl.packed = es == 2;
+  pl.vec = 4;
+  // whole tiles only: a lane's buckets lie a wave's width apart
+  if (b % (stream::kWave * pl.vec)) return pl;
+  pl.tiles = (uint32_t)(b / (stream::kWave * pl.vec));
+  if (pl.tiles > kMaxWaves) return pl;
+  pl.index_bits = 1;
+  while (pl.index_bits < 63 && (1ll << pl.index_bits) < n) ++pl.index_bits;
+  pl.split = 1;
+  pl.waves = pl.tiles;
+  pl.contig = pl.in_registers = true;
+  const size_t cand_bytes = (((size_t)k0 * es + 15) & ~(size_t)15) + (((size_t)k0 * 2 + 15) & ~(size_t)15);
+  pl.lds_bytes = cand_bytes > regs::kLdsBytes ? cand_bytes : regs::kLdsBytes;
+  pl.staged = (size_t)k * 8 <= kLdsBudget;
+  if (pl.staged && pl.lds_bytes < (size_t)k * 8) pl.lds_bytes = (size_t)k * 8;
+  pl.ok = true;
+  return pl;
+}
+
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned) {
   Plan pl{};
   pl.ok = false;
+  if (layout == ATK_BALANCED) return plan_short_buckets(rows, n, k0, j, k, dtype, aligned);
   // (a padded row is never reduced further: its callers keep every bucket)
   if (layout != ATK_INTERLEAVED) return pl;
   if (!aligned || rows > 0x7fffffffll) return pl;
@@ -171,7 +211,8 @@ bool describe_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stri
          std::to_string(j) + ", V=" + std::to_string(pl.vec) + ", pos" + (pl.pos16 ? "16" : "32") +
          ", PACKED=" + (pl.packed ? "1" : "0") + "> grid=" + std::to_string(rows) + " block=" +
          std::to_string(64 * pl.waves) + " tiles=" + std::to_string(pl.tiles) + " split=" + std::to_string(pl.split) +
-         " lds=" + std::to_string(pl.lds_bytes) + (pl.in_registers && pl.staged ? " staged" : "");
+         " lds=" + std::to_string(pl.lds_bytes) + (pl.in_registers && pl.staged ? " staged" : "") +
+         (pl.contig ? " short contiguous buckets" : "");
   return true;
 }
 

@@ -237,6 +237,13 @@ template <typename E, int J, int V> struct CmpQueue {
     }
     ATK_STATIC_FOR(v, V) { push<cmp_t, J, FILLED>(q[v], pos[v], c[v], p); } ATK_STATIC_END;
   }
+  // elements of sub-rows p and p + 1 of column VI
+  template <int VI, int FILLED> __device__ __forceinline__ void take_two(raw_t a, raw_t b, uint32_t p) {
+    const cmp_t ca = C::from_raw(a), cb = C::from_raw(b);
+    if constexpr (C::has_nan) nan_mask |= __ballot(__builtin_isunordered(ca, cb));
+    push<cmp_t, J, FILLED>(q[VI], pos[VI], ca, p);
+    push<cmp_t, J, (FILLED < J ? FILLED + 1 : J)>(q[VI], pos[VI], cb, p + 1);
+  }
   // one more element for column VI of a full queue, when `valid`
   template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
     const cmp_t c = C::from_raw(raw);
@@ -284,7 +291,7 @@ template <typename E, int J, int V> struct CmpQueue {
       } ATK_STATIC_END;
     } ATK_STATIC_END;
   }
-  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t) {}
+  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t, int64_t = 1) {}
   // exact order key of an entry (the queues are not poisoned)
   template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return E::key(C::to_raw(q[VI][SI])); }
   // A key cheap to get from an entry whose order is the selection order as far
@@ -462,6 +469,14 @@ template <typename E, int J, int V, bool SHIFTED = false, bool LEAN = !SHIFTED> 
       } ATK_STATIC_END;
     }
   }
+  // two elements of column VI as loaded in one dword: sub-row p (low half) and p + 1
+  template <int VI, int FILLED> __device__ __forceinline__ void take_two(uint32_t x, uint32_t p) {
+    constexpr int F = LEAN ? FILLED : J;
+    constexpr int F1 = F < J ? F + 1 : J;
+    const uint32_t keys = LEAN ? K::keys2_lean(x, screen) : K::keys2(x, screen);
+    insert_word<J, F>(q[VI], (keys << 16) | low_half(p));
+    insert_word<J, F1>(q[VI], (keys & 0xffff0000u) | low_half(p + 1));
+  }
   // one more element for column VI, when `valid` (the word 0 changes nothing)
   template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
     uint32_t scr = screen;
@@ -490,8 +505,9 @@ template <typename E, int J, int V, bool SHIFTED = false, bool LEAN = !SHIFTED> 
   // (entry words carry their whole order: any arrival order gives the same queue)
   __device__ __forceinline__ void fold_in_interleaved(const unsigned char* area, uint32_t lane) { fold_in(area, lane); }
   // Final entries with a zero key are re-read from the row to learn their sign.
-  // `col` is the lane's first column; call once, after the last fold, by live lanes.
-  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__ xr, int64_t b, int64_t col) {
+  // The element of sub-row p of the lane's v-th column is xr[p * b + col + v * step]
+  // (`col` is the lane's first column); call once, after the last fold, by live lanes.
+  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__ xr, int64_t b, int64_t col, int64_t step = 1) {
     if constexpr (K::zero_is_ambiguous) {
       bool any = false;
       ATK_STATIC_FOR(e, V * J) { any |= (q[e / J][e % J] >> 16) == K::kZeroKey; } ATK_STATIC_END;
@@ -500,7 +516,7 @@ template <typename E, int J, int V, bool SHIFTED = false, bool LEAN = !SHIFTED> 
         const uint32_t word = q[e / J][e % J];
         if ((word >> 16) == K::kZeroKey) {
           const uint32_t p = sub_row(word);
-          if (xr[(int64_t)p * b + col + e / J] == (raw_t)0x8000u) neg_zeros |= 1u << e;
+          if (xr[(int64_t)p * b + col + (e / J) * step] == (raw_t)0x8000u) neg_zeros |= 1u << e;
         }
       } ATK_STATIC_END;
     }
@@ -586,7 +602,7 @@ template <typename E, int J, int V> struct ByteQueue {
   }
   // (entry words carry their whole order: any arrival order gives the same queue)
   __device__ __forceinline__ void fold_in_interleaved(const unsigned char* area, uint32_t lane) { fold_in(area, lane); }
-  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t) {}
+  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__, int64_t, int64_t, int64_t = 1) {}
   template <int VI, int SI> __device__ __forceinline__ typename E::key_t key() const { return q[VI][SI] >> 24; }
   using sel_t = uint32_t;
   static constexpr int sel_bits = 32;
@@ -678,6 +694,13 @@ template <typename E, int J, int V> struct WideQueue {
     if constexpr (V % 2 != 0) nan_mask |= __ballot(__builtin_isunordered(c[V - 1], c[V - 1]));
     ATK_STATIC_FOR(v, V) { insert<FILLED>(q[v], word(c[v], np)); } ATK_STATIC_END;
   }
+  // elements of sub-rows p and p + 1 of column VI
+  template <int VI, int FILLED> __device__ __forceinline__ void take_two(raw_t a, raw_t b, uint32_t p) {
+    const float ca = __uint_as_float(a) + 0.0f, cb = __uint_as_float(b) + 0.0f;
+    nan_mask |= __ballot(__builtin_isunordered(ca, cb));
+    insert<FILLED>(q[VI], word(ca, ~p));
+    insert<(FILLED < J ? FILLED + 1 : J)>(q[VI], word(cb, ~(p + 1)));
+  }
   template <int VI> __device__ __forceinline__ void take_one(raw_t raw, uint32_t p, bool valid) {
     const float c = __uint_as_float(raw) + 0.0f;
     nan_mask |= __ballot(valid && __builtin_isunordered(c, c));
@@ -696,15 +719,16 @@ template <typename E, int J, int V> struct WideQueue {
   }
   __device__ __forceinline__ void fold_in_interleaved(const unsigned char* area, uint32_t lane) { fold_in(area, lane); }
   // Final entries with a zero element are re-read from the row to learn their
-  // sign.  `col` is the lane's first column; call once, after the last fold, by live lanes.
-  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__ xr, int64_t b, int64_t col) {
+  // sign (sub-row p of the lane's v-th column is xr[p * b + col + v * step]); call once,
+  // after the last fold, by live lanes.
+  __device__ __forceinline__ void fix_zeros(const raw_t* __restrict__ xr, int64_t b, int64_t col, int64_t step = 1) {
     bool any = false;
     ATK_STATIC_FOR(e, V * J) { any |= high(q[e / J][e % J]) == 0u; } ATK_STATIC_END;
     if (__ballot(any) == 0) return;
     ATK_STATIC_FOR(e, V * J) {
       if (high(q[e / J][e % J]) == 0u) {
         const uint32_t p = ~low(q[e / J][e % J]);
-        if (xr[(int64_t)p * b + col + e / J] == 0x80000000u) neg_zeros |= 1u << e;
+        if (xr[(int64_t)p * b + col + (e / J) * step] == 0x80000000u) neg_zeros |= 1u << e;
       }
     } ATK_STATIC_END;
   }
