@@ -104,31 +104,40 @@ REFERENCE_ROWS = (
        ("torch.topk", 256, 1 << 20, 65536, 1, 1)])
 
 
-def reference_rows(out_path: str, quick: bool) -> int:
+def reference_rows(out_path: str, quick: bool, only: list[int] | None = None, steady: bool = False) -> int:
+    """`steady`: 30 calls back to back per repetition over the resident inputs, which are filled once,
+    with no spin ahead of them: the rate of a loop of calls rather than of a call on fresh data."""
     device = torch.cuda.get_device_name()
+    rows = REFERENCE_ROWS if only is None else [REFERENCE_ROWS[i] for i in only]
     with open(out_path, "w") as out:
-        for name, batch, n, k, j, km in REFERENCE_ROWS:
+        for name, batch, n, k, j, km in rows:
             # two or three rotating inputs: together larger than the 256 MiB last-level cache
-            n_inner = 3 if batch * n * 2 < (1 << 30) else 2
-            xs = torch.zeros(n_inner, batch, n, device="cuda", dtype=torch.float16)
+            n_inputs = 3 if batch * n * 2 < (1 << 30) else 2
+            n_inner = 30 if steady else n_inputs
+            xs = torch.zeros(n_inputs, batch, n, device="cuda", dtype=torch.float16)
+            xs.normal_()
             if name == "approx_topk.topk":
-                call = lambda i: approx_topk(xs[i], k=k, dim=1, j=j, k_mult=km)[0]          # noqa: E731
+                call = lambda i: approx_topk(xs[i % n_inputs], k=k, dim=1, j=j, k_mult=km)[0]          # noqa: E731
             elif name == "bucketed_argmax.topk_torch":
-                call = lambda i: bucketed_argmax.topk_torch(xs[i], k=k, dim=1, interleaved=True)[0]   # noqa: E731
+                call = lambda i: bucketed_argmax.topk_torch(xs[i % n_inputs], k=k, dim=1, interleaved=True)[0]   # noqa: E731
             elif name == "bucketed_argmax.topk_triton":
-                call = lambda i: bucketed_argmax.topk_triton(xs[i], k=k, dim=1, interleaved=True)[0]  # noqa: E731
+                call = lambda i: bucketed_argmax.topk_triton(xs[i % n_inputs], k=k, dim=1, interleaved=True)[0]  # noqa: E731
             else:
-                call = lambda i: exact_topk(xs[i], k, 1)[0]                                  # noqa: E731
+                call = lambda i: exact_topk(xs[i % n_inputs], k, 1)[0]                                  # noqa: E731
             for graph in (False, True):
-                durations = time_calls(call, lambda: xs.normal_(), n_outer=8 if quick else 32, n_inner=n_inner,
-                                       graph=graph, n_warmup=4)
+                if steady:
+                    durations = time_calls(call, lambda: None, n_outer=4 if quick else 8, n_inner=n_inner,
+                                           graph=graph, n_warmup=2, hide_launch_cycles=0)
+                else:
+                    durations = time_calls(call, lambda: xs.normal_(), n_outer=8 if quick else 32, n_inner=n_inner,
+                                           graph=graph, n_warmup=4)
                 mean = sum(durations) / len(durations)
                 row = dict(method=name, args=dict(j=j, k_mult=km), batch_size=batch, topk_size=n, k=k,
-                           dtype="float16", hip_graphs=graph, n_inner=n_inner, duration=durations,
+                           dtype="float16", hip_graphs=graph, n_inner=n_inner, steady=steady, duration=durations,
                            input_GBps=2 * n * batch / mean / 1e9, device=device)
                 print(json.dumps(row), file=out, flush=True)
-                print(f"{name} fp16 [{batch}, {n}] k={k} j={j} k_mult={km} graph={graph}: "
-                      f"{mean * 1e6:.1f} us, {row['input_GBps']:.0f} GB/s", flush=True)
+                print(f"{name} fp16 [{batch}, {n}] k={k} j={j} k_mult={km} graph={graph}"
+                      f"{' steady' if steady else ''}: {mean * 1e6:.1f} us, {row['input_GBps']:.0f} GB/s", flush=True)
             del xs
             torch.cuda.empty_cache()
     return 0
@@ -141,9 +150,14 @@ def main() -> int:
     ap.add_argument("--no-compile", action="store_true", help="leave out the torch.compile variants")
     ap.add_argument("--reference-rows", action="store_true",
                     help="the shapes of the reference's own recorded measurements (fp16) instead of the grid")
+    ap.add_argument("--only", default=None,
+                    help="with --reference-rows: comma-separated numbers of the rows to time (for a profiler run)")
+    ap.add_argument("--steady", action="store_true",
+                    help="with --reference-rows: 30 calls back to back per repetition, inputs filled once, no spin")
     args = ap.parse_args()
     if args.reference_rows:
-        return reference_rows(args.out, args.quick)
+        only = None if args.only is None else [int(i) for i in args.only.split(",")]
+        return reference_rows(args.out, args.quick, only, args.steady)
 
     # (name, function, arguments, compiled): as the reference does (benchmarks/measure_speed.py:66-71,
     # 292-296), the approximate top-k and the torch-level arg-max are also timed under

@@ -25,15 +25,16 @@ def main(path: str) -> int:
         regime = "k=64" if row["k"] == 64 else f"k=n/{row['topk_size'] // row['k']}"
         key = (row["batch_size"], regime, row["hip_graphs"])
         gbps = BYTES[row["dtype"]] * row["topk_size"] * row["batch_size"] / mean / 1e9
-        tables[key][row["topk_size"]][row["method"]] = (gbps, mean * 1e6)
-        if row["method"] not in methods:
-            methods.append(row["method"])
+        method = row["method"] + (" compiled" if row.get("compile") else "")  # under torch.compile: a column of its own
+        tables[key][row["topk_size"]][method] = (gbps, mean * 1e6)
+        if method not in methods:
+            methods.append(method)
     for (batch, regime, graphs), by_n in sorted(tables.items()):
         print(f"\nbatch {batch}, {regime}, HIP graphs {'on' if graphs else 'off'}: GB/s read (us per call)")
-        print("n".rjust(8) + "".join(m.rjust(30) for m in methods))
+        print("n".rjust(8) + "".join(m.replace("approx_topk.topk", "approx").replace("bucketed_argmax.", "").rjust(22) for m in methods))
         for n in sorted(by_n):
             cells = [by_n[n].get(m) for m in methods]
-            print(str(n).rjust(8) + "".join(("%.0f (%.1f)" % c if c else "-").rjust(30) for c in cells))
+            print(str(n).rjust(8) + "".join(("%.0f (%.1f)" % c if c else "-").rjust(22) for c in cells))
     return 0
 
 
