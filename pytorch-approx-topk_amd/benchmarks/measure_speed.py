@@ -15,7 +15,8 @@ per-call durations in seconds; input bandwidth is dtype_bytes * n * batch / mean
 
     python pytorch-approx-topk_amd/benchmarks/measure_speed.py [--out results.jsonl] [--quick]
 
-`--reference-rows` times instead the shapes of the measurements the reference keeps of itself
+`--shapes` times given shapes in steady state (calls back to back); `--reference-rows` times instead the
+shapes of the measurements the reference keeps of itself
 (fp16, batch 256 or 1, an H100 PCIe: notebooks/data/generic2/measure_speed_approx_finer_multi2.jsonl
 and measure_speed_exact_finer.jsonl), for orientation beside those figures.
 """
@@ -143,6 +144,47 @@ def reference_rows(out_path: str, quick: bool, only: list[int] | None = None, st
     return 0
 
 
+DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16, "int32": torch.int32,
+          "int16": torch.int16, "uint8": torch.uint8}
+
+
+def time_shapes(spec: str, out_path: str) -> int:
+    """Steady-state time per call of `approx_topk.topk` at given shapes, beside the planner's description.
+
+    `spec`: shapes separated by ';', each dtype:rows:n:k:j:k_mult[:layout[:data]] with layout `interleaved`
+    (default) or `contiguous` and data `normal` (default) or `sparse` (relu(N(0,1) - 2.5): 0.6 % of the elements
+    are positive, the rest zeros; with buckets of around a hundred elements most candidates are zeros, and so is
+    the cut: thousands of candidates of one key, told apart by their indices)."""
+    from approx_topk import _native
+    device = torch.cuda.get_device_name()
+    with open(out_path, "w") as out:
+        for item in spec.split(";"):
+            f = item.strip().split(":")
+            dtype, (rows, n, k, j, km) = DTYPES[f[0]], (int(v) for v in f[1:6])
+            interleaved = len(f) < 7 or f[6] == "interleaved"
+            data = f[7] if len(f) > 7 else "normal"
+            n_inputs = max(2, min(8, (1 << 29) // max(1, rows * n * torch.empty(0, dtype=dtype).element_size())))
+            base = torch.randn(n_inputs, rows, n, device="cuda")
+            if data == "sparse":
+                base = torch.relu(base - 2.5)
+            xs = (base * (30 if not dtype.is_floating_point else 1)).to(dtype)
+            del base
+            call = lambda i: approx_topk(xs[i % n_inputs], k=k, dim=1, j=j, k_mult=km, interleaved=interleaved)[0]  # noqa: E731
+            durations = time_calls(call, lambda: None, n_outer=8, n_inner=30, graph=False, n_warmup=2,
+                                   hide_launch_cycles=0)
+            mean = sum(durations) / len(durations)
+            kernels = _native.describe(xs[0], k * km, j, k, layout=_native.INTERLEAVED if interleaved else 1)
+            row = dict(method="approx_topk.topk", args=dict(j=j, k_mult=km, interleaved=interleaved), data=data,
+                       batch_size=rows, topk_size=n, k=k, dtype=f[0], duration=durations, kernels=kernels,
+                       input_GBps=xs.element_size() * n * rows / mean / 1e9, device=device)
+            print(json.dumps(row), file=out, flush=True)
+            print(f"{f[0]} [{rows}, {n}] k={k} j={j} k_mult={km} {'interleaved' if interleaved else 'contiguous'} "
+                  f"{data}: {mean * 1e6:.1f} us, {row['input_GBps']:.0f} GB/s | {kernels}", flush=True)
+            del xs
+            torch.cuda.empty_cache()
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default="measure_speed.jsonl")
@@ -154,7 +196,11 @@ def main() -> int:
                     help="with --reference-rows: comma-separated numbers of the rows to time (for a profiler run)")
     ap.add_argument("--steady", action="store_true",
                     help="with --reference-rows: 30 calls back to back per repetition, inputs filled once, no spin")
+    ap.add_argument("--shapes", default=None,
+                    help="time these shapes instead: dtype:rows:n:k:j:k_mult[:interleaved|contiguous[:normal|sparse]];...")
     args = ap.parse_args()
+    if args.shapes:
+        return time_shapes(args.shapes, args.out)
     if args.reference_rows:
         only = None if args.only is None else [int(i) for i in args.only.split(",")]
         return reference_rows(args.out, args.quick, only, args.steady)
