@@ -191,11 +191,11 @@ __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80))) 
 // ---------------------------------------------------------------------------
 namespace regs = select::regs;
 
-// Stage 1 of a row whose buckets are runs of `m` adjacent elements of 16 to 64
+// Stage 1 of a row whose buckets are runs of `m` adjacent elements of 16 to 256
 // bytes each (contiguous layout, every bucket as long).  A lane takes V buckets
 // kWave apart, `first` the first of them, so that the lanes of a wave load from
-// adjacent buckets, and loads a bucket whole, 16 bytes at a time, before it
-// feeds it to the bucket's queue with the place within the bucket as the sub-row
+// adjacent buckets, and loads a bucket whole (64 bytes of it at a time), 16
+// bytes a load, before it feeds it to the bucket's queue with the place within the bucket as the sub-row
 // number: the loads of a wave then cover a stretch of the row back to back.
 // (With the lane's buckets side by side, lanes 128-256 bytes apart, and with one
 // load per bucket at a time, so that the second 16 bytes of a cache line are
@@ -207,7 +207,7 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
                                                    int64_t first, Queue& queue) {
   using raw_t = typename E::raw_t;
   constexpr int EPL = 16 / (int)sizeof(raw_t);  // elements per load
-  constexpr int kMaxLoads = 4;                  // a bucket is at most 64 bytes
+  constexpr int kMaxLoads = 4;                  // loads of a bucket issued together
   static_assert(EPL >= J && EPL % 2 == 0, "the first load of a bucket fills its queue");
   using Load = stream::Pack<raw_t, EPL>;
   const raw_t* next = xr + first * (int64_t)m;
@@ -221,22 +221,40 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
     }
     next += apart;
   };
-  auto feed = [&](auto v_c, const Load (&buf)[kMaxLoads]) __attribute__((always_inline)) {
+  // the loads `buf` of bucket v: elements at + c * EPL .. of the bucket, c = 0 .. kMaxLoads - 1
+  auto feed_loads = [&](auto v_c, auto first_c, const Load (&buf)[kMaxLoads], uint32_t at, uint32_t count)
+      __attribute__((always_inline)) {
     constexpr int v = decltype(v_c)::value;
+    constexpr bool kFirst = decltype(first_c)::value;  // the bucket's first loads: its queue fills
     ATK_STATIC_FOR(c, kMaxLoads) {
-      if (c == 0 || (uint32_t)c < loads) {
+      if (c == 0 || (uint32_t)c < count) {
         ATK_STATIC_FOR(d, EPL / 2) {
-          constexpr int kFilled = (c == 0 && 2 * d < J) ? 2 * d : J;
+          constexpr int kFilled = (kFirst && c == 0 && 2 * d < J) ? 2 * d : J;
           if constexpr (PACKED) {
             uint32_t x;
             __builtin_memcpy(&x, &buf[c].e[2 * d], 4);
-            queue.template take_two<v, kFilled>(x, c * EPL + 2 * d);
+            queue.template take_two<v, kFilled>(x, at + c * EPL + 2 * d);
           } else {
-            queue.template take_two<v, kFilled>(buf[c].e[2 * d], buf[c].e[2 * d + 1], c * EPL + 2 * d);
+            queue.template take_two<v, kFilled>(buf[c].e[2 * d], buf[c].e[2 * d + 1], at + c * EPL + 2 * d);
           }
         } ATK_STATIC_END;
       }
     } ATK_STATIC_END;
+  };
+  auto feed = [&](auto v_c, const Load (&buf)[kMaxLoads]) __attribute__((always_inline)) {
+    constexpr int v = decltype(v_c)::value;
+    feed_loads(v_c, std::true_type{}, buf, 0u, loads);
+    // a bucket of more than 64 bytes: the rest of it, kMaxLoads loads at a time
+    const raw_t* rest = xr + (first + (int64_t)v * kWave) * (int64_t)m;
+#pragma nounroll
+    for (uint32_t c0 = kMaxLoads; c0 < loads; c0 += kMaxLoads) {
+      Load more[kMaxLoads];
+#pragma unroll
+      for (int c = 0; c < kMaxLoads; ++c) {
+        if (c == 0 || c0 + (uint32_t)c < loads) more[c] = stream::load_pack<raw_t, EPL>(rest + (c0 + c) * EPL);
+      }
+      feed_loads(v_c, std::false_type{}, more, c0 * EPL, loads - c0);
+    }
   };
   if constexpr (AHEAD) {
     Load buf[2][kMaxLoads];
@@ -258,7 +276,7 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
 // (eight waves per SIMD: four 8-wave workgroups per CU); what does not fit is
 // spilled where the pressure peaks, in the rarely taken LDS path.
 // CONTIG: the row's buckets are contiguous runs of g.full_rows elements of at
-// most 64 bytes (no remainder, whole tiles, one wave per tile).  The scan differs,
+// most 256 bytes (no remainder, whole tiles, one wave per tile).  The scan differs,
 // the way an index is put together, and which buckets a lane holds: V buckets
 // kWave apart (bucket_of), so that a wave's candidates in their order are those
 // of every lane's first bucket, then of every lane's second, ...

@@ -29,15 +29,19 @@ constexpr size_t kLdsBudgetLarge = 128 * 1024;
 constexpr uint32_t kMaxWaves = 8;
 // Corners in which the two-kernel path may be the faster one (see make_plan).
 constexpr int64_t kManyRows = 1024, kAllCus = 256;
+// Longest contiguous bucket (bytes) the register kernel takes.
+constexpr int64_t kShortBucket = 256;
 constexpr size_t kShortRow = 128 * 1024, kLongRow = 512 * 1024;
 }  // namespace
 
-// Contiguous buckets, all of one length of 16 to 64 bytes (a quarter to a
-// sixteenth of the row's elements become candidates), elements of two or four
-// bytes: a lane of the register kernel loads its four buckets whole.  The
+// Contiguous buckets, all of one length of 16 to kShortBucket bytes, elements of
+// two or four bytes: a lane of the register kernel loads its four buckets whole.  The
 // alternative is a stage-1 kernel that copies spans of buckets through LDS and
 // parks the candidates in HBM for a stand-alone select: fp16 [1024, 32768]
-// k=2048 j=4 k_mult=4 68.6 us that way.
+// k=2048 j=4 k_mult=4 (buckets of 32 bytes) 68.6 us that way against 35; buckets of
+// 128 bytes fp16 [256, 131072] k0=8192 39.2 against 33.3 us, fp32 [64, 32768] k0=2048
+// 17.4 against 12.7 us; of 256 bytes fp16 [256, 262144] k0=8192 57.6 against 49.4 us,
+// [1024, 131072] 109.9 against 110.3 us.
 static Plan plan_short_buckets(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int dtype, bool aligned) {
   Plan pl{};
   pl.ok = false;
@@ -45,11 +49,14 @@ static Plan plan_short_buckets(int64_t rows, int64_t n, int64_t k0, int j, int64
   if (k0 <= 0 || k <= 0 || k >= k0 || j < 1 || j > 4 || k0 % j) return pl;
   const int es = elem_bytes(dtype);
   if (es != 2 && es != 4) return pl;
-  if (rows < kMinRows && (size_t)n * es > kSoloRow) return pl;
+  // fewer rows than CUs: only rows one workgroup reads in a few microseconds (fp32 [130, 131072]
+  // with 2048 buckets of 256 bytes: 38.4 us here against 32.4 through two kernels, whose stage 1
+  // has sixteen workgroups per row)
+  if (rows < kAllCus && (size_t)n * es > kSoloRow) return pl;
   const int64_t b = k0 / j;
   if (n % b) return pl;
   const int64_t m = n / b;
-  if ((m * es) % 16 || m * es > 64 || m < j) return pl;
+  if ((m * es) % 16 || m * es > kShortBucket || m < j) return pl;
   pl.full_rows = (uint32_t)m;
   pl.pos16 = true;
   pl.packed = es == 2;

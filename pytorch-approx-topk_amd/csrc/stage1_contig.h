@@ -59,6 +59,7 @@ struct Geom {
   uint32_t slabs;        // > 1 (only with chunks > 1): workgroups sharing a bucket's chunks
   uint32_t slab_chunks;  // least chunks per slab: slab s takes chunks [s * chunks / slabs, (s + 1) * chunks / slabs)
   uint32_t fast;         // the shape allows scan_even (see there)
+  uint32_t whole;        // the shape allows whole_bucket_kernel (see there)
   uint32_t wide_out;     // the outputs allow 16-byte stores (filled in at launch)
 };
 
@@ -422,6 +423,130 @@ __global__ __launch_bounds__(kThreads) void contig_kernel(const typename E::raw_
     __syncthreads();
     scan_buckets<E, J, V, KeyForm<E>>(xr, values, indices, partial, row, group, g, contig_lds);
   }
+}
+
+// Buckets of one length of 16 to kWholeBucket bytes (no remainder, rows that allow
+// 16-byte loads, elements of two or four bytes): a lane per bucket.  The lane loads
+// its bucket whole, 64 bytes of it at a time, 16 bytes a load -- neighbouring lanes
+// hold neighbouring buckets, so the loads of a wave cover a stretch of the row back
+// to back -- feeds it to a one-column register queue of the streaming kernel with
+// the place within the bucket as the sub-row number, and writes the bucket's J
+// entries; nothing goes through LDS and a row needs no workgroup of its own.  A NaN
+// (a wave that met one) sends the wave's lanes through their buckets again with
+// order keys.  Buckets are numbered row after row: lane t of workgroup w takes
+// bucket w * kThreads + t of the rows * b there are.
+constexpr uint32_t kWholeBucket = 64;
+
+template <typename E, int J, bool PACKED>
+__global__ __launch_bounds__(kThreads) void whole_bucket_kernel(const typename E::raw_t* __restrict__ x,
+                                                                typename E::raw_t* __restrict__ values,
+                                                                const IndexOut indices, const Geom g,
+                                                                int64_t buckets) {
+  using raw_t = typename E::raw_t;
+  using Queue = stream::QueueFor<E, J, 1, PACKED>;
+  constexpr int EPL = 16 / (int)sizeof(raw_t);  // elements per load
+  constexpr int kMaxLoads = 4;                  // loads of a bucket issued together
+  static_assert(EPL >= J && EPL % 2 == 0, "the first load of a bucket fills its queue");
+  using Load = Pack<raw_t, EPL>;
+
+  const int64_t at = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const bool has = at < buckets;
+  const int64_t mine = has ? at : buckets - 1;  // idle lanes go through the last bucket and write nothing
+  int64_t row;
+  uint32_t c;
+  if (buckets <= 0xffffffffll) {
+    const uint32_t row32 = (uint32_t)mine / g.b;
+    row = row32;
+    c = (uint32_t)mine - row32 * g.b;
+  } else {
+    row = mine / g.b;
+    c = (uint32_t)(mine - row * g.b);
+  }
+  const raw_t* xr = x + row * g.row_stride;
+  const raw_t* bucket = xr + (int64_t)c * g.m;
+  const uint32_t loads = __builtin_amdgcn_readfirstlane(g.m / EPL);
+
+  Queue queue;
+  queue.reset();
+  auto feed = [&](auto first_c, const Load (&buf)[kMaxLoads], uint32_t from, uint32_t count)
+      __attribute__((always_inline)) {
+    constexpr bool kFirst = decltype(first_c)::value;  // the bucket's first loads: its queue fills
+    ATK_STATIC_FOR(l, kMaxLoads) {
+      if (l == 0 || (uint32_t)l < count) {
+        ATK_STATIC_FOR(d, EPL / 2) {
+          constexpr int kFilled = (kFirst && l == 0 && 2 * d < J) ? 2 * d : J;
+          if constexpr (PACKED) {
+            uint32_t pair;
+            __builtin_memcpy(&pair, &buf[l].e[2 * d], 4);
+            queue.template take_two<0, kFilled>(pair, from + l * EPL + 2 * d);
+          } else {
+            queue.template take_two<0, kFilled>(buf[l].e[2 * d], buf[l].e[2 * d + 1], from + l * EPL + 2 * d);
+          }
+        } ATK_STATIC_END;
+      }
+    } ATK_STATIC_END;
+  };
+  {
+    Load buf[kMaxLoads];
+#pragma unroll
+    for (int l = 0; l < kMaxLoads; ++l) {
+      if (l == 0 || (uint32_t)l < loads) buf[l] = stream::load_pack<raw_t, EPL>(bucket + l * EPL);
+    }
+    feed(std::true_type{}, buf, 0u, loads);
+  }
+#pragma nounroll
+  for (uint32_t l0 = kMaxLoads; l0 < loads; l0 += kMaxLoads) {
+    Load buf[kMaxLoads];
+#pragma unroll
+    for (int l = 0; l < kMaxLoads; ++l) {
+      if (l == 0 || l0 + (uint32_t)l < loads) buf[l] = stream::load_pack<raw_t, EPL>(bucket + (l0 + l) * EPL);
+    }
+    feed(std::false_type{}, buf, l0 * EPL, loads - l0);
+  }
+
+  const int64_t o = (row * g.b + c) * J;
+  const int64_t first_index = (int64_t)c * g.m;
+  if (queue.poisoned()) {  // (wave-uniform)
+    raw_t qv[J];
+    uint32_t qp[J];
+    stream::clear_exact<E, J>(qv, qp);
+    for (uint32_t p = 0; p < g.m; ++p) stream::push_exact<E, J>(qv, qp, bucket[p], p);
+    if (!has) return;
+#pragma unroll
+    for (int sl = 0; sl < J; ++sl) {
+      if (values != nullptr) values[o + sl] = qv[sl];
+      indices.put(o + sl, first_index + qp[sl]);
+    }
+    return;
+  }
+  queue.fix_zeros(xr, 1, first_index, 0);
+  if (!has) return;
+  if constexpr (J == 2 || J == 4) {
+    if (g.wide_out != 0) {  // the outputs allow whole-bucket stores
+      if (values != nullptr) {
+        Pack<raw_t, J> pv;
+        ATK_STATIC_FOR(sl, J) { pv.e[sl] = queue.template raw<0, sl>(); } ATK_STATIC_END;
+        *reinterpret_cast<Pack<raw_t, J>*>(values + o) = pv;
+      }
+      if (indices.narrow) {
+        Pack<int32_t, J> pi;
+        ATK_STATIC_FOR(sl, J) { pi.e[sl] = (int32_t)(first_index + queue.template position<0, sl>()); } ATK_STATIC_END;
+        *reinterpret_cast<Pack<int32_t, J>*>(static_cast<int32_t*>(indices.base) + o) = pi;
+      } else {
+        ATK_STATIC_FOR(t, J / 2) {
+          Pack<int64_t, 2> pi;
+          pi.e[0] = first_index + queue.template position<0, 2 * t>();
+          pi.e[1] = first_index + queue.template position<0, 2 * t + 1>();
+          reinterpret_cast<Pack<int64_t, 2>*>(static_cast<int64_t*>(indices.base) + o)[t] = pi;
+        } ATK_STATIC_END;
+      }
+      return;
+    }
+  }
+  ATK_STATIC_FOR(sl, J) {
+    if (values != nullptr) values[o + sl] = queue.template raw<0, sl>();
+    indices.put(o + sl, first_index + queue.template position<0, sl>());
+  } ATK_STATIC_END;
 }
 
 // Combines the `slabs` partial results of every bucket: one wave per bucket,

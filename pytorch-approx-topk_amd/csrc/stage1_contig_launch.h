@@ -24,6 +24,20 @@ template <typename E, int J>
 static int launch_j(const Plan& pl, const Geom& g, const typename E::raw_t* x, int64_t rows,
                     typename E::raw_t* values, IndexOut indices, void* ws, hipStream_t stream) {
   constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
+  if (g.whole != 0) {
+    constexpr int ES = (int)sizeof(typename E::raw_t);
+    if constexpr (ES == 2 || ES == 4) {
+      const int64_t buckets = rows * (int64_t)g.b;
+      const int64_t groups = (buckets + kThreads - 1) / kThreads;
+      if (groups > 0x7fffffffll) return ATK_ERR_TOO_LARGE;
+      constexpr bool kPacked = ES == 2 && stream::PackedKey<E>::available;
+      hipLaunchKernelGGL((whole_bucket_kernel<E, J, kPacked>), dim3((unsigned)groups), dim3(kThreads), 0, stream, x,
+                         values, indices, g, buckets);
+      return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
+    } else {
+      return ATK_ERR_ARG;  // the planner never asks for it
+    }
+  }
   return pl.vec > 1 ? launch_one<E, J, VF>(pl, g, x, rows, values, indices, ws, stream)
                     : launch_one<E, J, 1>(pl, g, x, rows, values, indices, ws, stream);
 }
@@ -34,6 +48,7 @@ int launch_typed(const Plan& pl, const void* x, int64_t rows, int64_t row_stride
   using raw_t = typename E::raw_t;
   Geom g = pl.geom;
   g.row_stride = row_stride;
+  // (whole_bucket_kernel stores a bucket's J values at once: J * sizeof(raw_t) bytes, at most 16)
   g.wide_out = ((uintptr_t)values % 16 == 0 && (uintptr_t)indices.base % 16 == 0) ? 1u : 0u;
   const raw_t* xs = static_cast<const raw_t*>(x);
   raw_t* vs = static_cast<raw_t*>(values);

@@ -82,6 +82,15 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
       if (pl.lds_bytes < even_bytes) pl.lds_bytes = (even_bytes + 15) / 16 * 16;
     }
   }
+  // whole_bucket_kernel: a lane per bucket, no LDS
+  g.whole = 0;
+  if (pl.vec > 1 && (es == 2 || es == 4) && r == 0 && (int64_t)b * m == n && (m * es) % 16 == 0 &&
+      m * es <= (int64_t)kWholeBucket) {
+    g.whole = 1;
+    g.slabs = 1;
+    pl.ws_bytes = 0;
+    pl.lds_bytes = 0;
+  }
   if (pl.lds_bytes > 64 * 1024) return pl;
   pl.ok = true;
   return pl;
@@ -105,6 +114,11 @@ bool describe_stage1_contig(const void* x, int64_t rows, int64_t n, int64_t row_
   const bool aligned = ((uintptr_t)x % 16 == 0) && (row_stride % vf == 0);
   const contig::Plan pl = contig::make_plan(rows, n, k0, j, layout, dtype, aligned);
   if (!pl.ok) return false;
+  if (pl.geom.whole) {
+    out += "whole_bucket_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + "> grid=" +
+           std::to_string((rows * (int64_t)pl.geom.b + contig::kThreads - 1) / contig::kThreads) + " block=256";
+    return true;
+  }
   out += "contig_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + ", V=" +
          std::to_string(pl.vec) + "> grid=" + std::to_string(rows * (int64_t)pl.geom.groups) + " block=256 chunks=" +
          std::to_string(pl.geom.chunks) + " slabs=" + std::to_string(pl.geom.slabs) +

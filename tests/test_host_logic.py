@@ -41,10 +41,10 @@ def test_workspace_of_one_call_depends_on_the_address():
     # k == k0: stage 1 alone
     assert L.atk_topk_workspace_bytes_at(4096, 512, 32768, 32768, 1024, 1, 1024, 0, 1) == \
         L.atk_topk_workspace_bytes(512, 32768, 1024, 1, 1024, 0, 1)
-    # contiguous buckets: one kernel for buckets of up to 64 bytes (here 32 elements), else two
+    # contiguous buckets: one kernel for buckets of up to 256 bytes (here 32 elements), else two
     assert L.atk_topk_workspace_bytes_at(4096, 512, 32768, 32768, 1024, 1, 256, 1, 1) == 0
-    assert L.atk_topk_workspace_bytes_at(4096, 512, 32768, 32768, 512, 1, 256, 1, 1) == \
-        L.atk_topk_workspace_bytes(512, 32768, 512, 1, 256, 1, 1) > 0
+    assert L.atk_topk_workspace_bytes_at(4096, 512, 1 << 18, 1 << 18, 1024, 1, 256, 1, 1) == \
+        L.atk_topk_workspace_bytes(512, 1 << 18, 1024, 1, 256, 1, 1) > 0
 
 
 def test_native_argument_checks_need_no_gpu():
@@ -111,7 +111,7 @@ def test_describe_names_the_planned_kernels():
     # a misaligned input: scalar loads, and two kernels instead of the fused one
     odd = describe(1024, 32768, 1, 2048, 4, 4, x=4098)
     assert odd.startswith("stream_kernel<f16, J=4, V=1") and "select_kernel<f16" in odd
-    # contiguous buckets of 16-64 bytes with a second stage: one kernel too; longer buckets, a bucket
+    # contiguous buckets of 16-256 bytes with a second stage: one kernel too; longer buckets, a bucket
     # count that does not fill whole column tiles, or a row with a remainder: two kernels
     def contiguous(rows, n, code, k, j, k_mult):
         buf = ctypes.create_string_buffer(1024)
@@ -121,8 +121,13 @@ def test_describe_names_the_planned_kernels():
     assert short.startswith("fused_regs_kernel<f16, J=4, V=4, pos16, PACKED=1> grid=1024 block=512")
     assert short.endswith("short contiguous buckets") and "select" not in short
     assert contiguous(1024, 32768, 0, 2048, 4, 4).endswith("short contiguous buckets")   # fp32: 64 bytes
-    assert contiguous(1024, 65536, 0, 2048, 4, 4).startswith("contig_kernel<f32")         # 128 bytes
+    assert contiguous(1024, 65536, 0, 2048, 4, 4).endswith("short contiguous buckets")   # 128 bytes
+    assert contiguous(256, 1 << 18, 0, 2048, 4, 4).startswith("contig_kernel<f32")        # 512 bytes
+    # no second stage: a lane per bucket up to 64 bytes, spans of buckets through LDS beyond
     assert contiguous(1024, 32768, 1, 2048, 4, 1).startswith("contig_kernel<f16")         # 128 bytes
+    assert contiguous(1024, 32768, 1, 4096, 4, 1).startswith("whole_bucket_kernel<f16, J=4> grid=4096 block=256")
+    assert contiguous(16384, 1024, 1, 64, 2, 1).startswith("whole_bucket_kernel<f16, J=2> grid=2048 ")
+    assert contiguous(16, 1028, 0, 256, 1, 1).startswith("contig_kernel<f32")             # 1028 = 4 * 256 + 4
     assert contiguous(16, 3072, 1, 64, 2, 4).startswith("contig_kernel<f16")              # 128 buckets
     assert contiguous(16, 8200, 1, 512, 2, 2).startswith("contig_kernel<f16")             # 8200 = 16 * 512 + 8
     assert contiguous(1024, 32768, 4, 2048, 4, 4).startswith("contig_kernel<u8")          # 1-byte elements
