@@ -128,7 +128,8 @@ def test_describe_names_the_planned_kernels():
     assert contiguous(1024, 32768, 1, 4096, 4, 1).startswith("whole_bucket_kernel<f16, J=4> grid=4096 block=256")
     assert contiguous(16384, 1024, 1, 64, 2, 1).startswith("whole_bucket_kernel<f16, J=2> grid=2048 ")
     assert contiguous(16, 1028, 0, 256, 1, 1).startswith("contig_kernel<f32")             # 1028 = 4 * 256 + 4
-    assert contiguous(16, 3072, 1, 64, 2, 4).startswith("contig_kernel<f16")              # 128 buckets
+    two = contiguous(16, 3072, 1, 64, 2, 4)                                               # 128 buckets: two kernels
+    assert two.startswith("whole_bucket_kernel<f16, J=2> grid=8 ") and "select_kernel<f16" in two
     assert contiguous(16, 8200, 1, 512, 2, 2).startswith("contig_kernel<f16")             # 8200 = 16 * 512 + 8
     assert contiguous(1024, 32768, 4, 2048, 4, 4).startswith("contig_kernel<u8")          # 1-byte elements
     # truncation and argument checks
