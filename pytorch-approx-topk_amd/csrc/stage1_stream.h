@@ -874,6 +874,107 @@ __device__ __forceinline__ void emit(const Geom& g, const Sink<typename E::raw_t
   }
 }
 
+// The same for final results, by the one wave that holds a tile's queues, with
+// every store instruction covering 1 KiB of adjacent bytes.  Written as above, a
+// store instruction sends 64 separate 16-byte pieces to L2, a lane's stretch of
+// output (V * J entries) apart: fp16 [128, 2^20] k=262144 j=4, 32 entries a lane,
+// took 188 us that way and takes 109 us this way, [256, 2^20] k=65536 j=4 147 -> 135 us
+// and j=2 132 -> 118 us, uint8 [128, 2^20] k=65536 j=2 50 -> 42 us, fp32 k=262144 j=4
+// 177 -> 165 us; with eight 4-byte entries a lane (fp32, j=2) it makes no difference.
+// The lanes park their entries in LDS -- the elements in one array, the sub-row
+// numbers in another, a lane's stretch 16 bytes further on than a power of two
+// from the next lane's for the banks -- and read them back in the order of the
+// output.  `col0`: the tile's first column; lanes beyond the row's last column
+// hold nothing that is read.  One wave: its LDS accesses complete in program
+// order, so nothing waits on a barrier.
+template <typename E, int J, int V>
+struct Transposed {
+  using raw_t = typename E::raw_t;
+  static constexpr int NC = V * J;                           // entries of a lane
+  static constexpr int kPerStore = 16 / (int)sizeof(raw_t);  // elements in 16 bytes
+  // whole 16-byte pieces on both sides, elements of up to four bytes
+  static constexpr bool available = V > 1 && sizeof(raw_t) <= 4 && NC % 4 == 0 && NC % kPerStore == 0;
+  static constexpr size_t kRawPitch = (size_t)NC * sizeof(raw_t) + 16;  // bytes from lane to lane
+  static constexpr size_t kPosPitch = (size_t)NC * 4 + 16;
+  static constexpr size_t kPosArea = kWave * kRawPitch;                 // where the sub-row numbers start
+  static constexpr size_t kBytes = kPosArea + kWave * kPosPitch;
+};
+
+template <typename E, int J, int V, typename Queue>
+__device__ __forceinline__ void emit_transposed(const Geom& g, const Sink<typename E::raw_t>& out, int64_t row,
+                                                int64_t col0, uint32_t lane, const Queue& queue,
+                                                unsigned char* lds) {
+  using raw_t = typename E::raw_t;
+  using T = Transposed<E, J, V>;
+  constexpr int NC = T::NC, kPerStore = T::kPerStore;
+  static_assert(T::available, "see Transposed");
+  unsigned char* raws = lds;
+  unsigned char* poss = lds + T::kPosArea;
+  if (out.values != nullptr) {
+    ATK_STATIC_FOR(t, NC / kPerStore) {
+      Pack<raw_t, kPerStore> pv;
+      ATK_STATIC_FOR(u, kPerStore) {
+        constexpr int e = t * kPerStore + u;
+        pv.e[u] = queue.template raw<e / J, e % J>();
+      } ATK_STATIC_END;
+      *reinterpret_cast<Pack<raw_t, kPerStore>*>(raws + lane * T::kRawPitch + 16 * t) = pv;
+    } ATK_STATIC_END;
+  }
+  ATK_STATIC_FOR(t, NC / 4) {
+    uint32_t w[4];
+    ATK_STATIC_FOR(u, 4) {
+      constexpr int e = t * 4 + u;
+      w[u] = queue.template position<e / J, e % J>();
+    } ATK_STATIC_END;
+    *reinterpret_cast<uint4*>(poss + lane * T::kPosPitch + 16 * t) = make_uint4(w[0], w[1], w[2], w[3]);
+  } ATK_STATIC_END;
+
+  const int64_t left = (g.b - col0) * J;  // entries from this tile's first to the row's last
+  const uint32_t valid = left < (int64_t)(kWave * NC) ? (uint32_t)left : (uint32_t)(kWave * NC);
+  const int64_t o = (row * g.b + col0) * J;
+  if (out.values != nullptr) {
+    ATK_STATIC_FOR(t, NC / kPerStore) {
+      const uint32_t i = t * (kWave * kPerStore) + lane * kPerStore;  // (valid is a multiple of kPerStore)
+      if (i < valid) {
+        const Pack<raw_t, kPerStore> pv = *reinterpret_cast<const Pack<raw_t, kPerStore>*>(
+            raws + (i / NC) * T::kRawPitch + (i % NC) * sizeof(raw_t));
+        *reinterpret_cast<Pack<raw_t, kPerStore>*>(out.values + o + i) = pv;
+      }
+    } ATK_STATIC_END;
+  }
+  auto pos_at = [&](uint32_t i) __attribute__((always_inline)) -> const unsigned char* {
+    return poss + (i / NC) * T::kPosPitch + (i % NC) * 4;
+  };
+  auto index_of = [&](uint32_t i, uint32_t sub_row) __attribute__((always_inline)) -> int64_t {
+    return col0 + (int64_t)(i / J) + (int64_t)sub_row * g.b;
+  };
+  if (out.indices.narrow) {
+    int32_t* oi = static_cast<int32_t*>(out.indices.base) + o;
+    ATK_STATIC_FOR(t, NC / 4) {
+      const uint32_t i = t * (kWave * 4) + lane * 4;
+      if (i < valid) {
+        const uint4 a = *reinterpret_cast<const uint4*>(pos_at(i));
+        Pack<int32_t, 4> pi;
+        pi.e[0] = (int32_t)index_of(i, a.x); pi.e[1] = (int32_t)index_of(i + 1, a.y);
+        pi.e[2] = (int32_t)index_of(i + 2, a.z); pi.e[3] = (int32_t)index_of(i + 3, a.w);
+        *reinterpret_cast<Pack<int32_t, 4>*>(oi + i) = pi;
+      }
+    } ATK_STATIC_END;
+  } else {
+    int64_t* oi = static_cast<int64_t*>(out.indices.base) + o;
+    ATK_STATIC_FOR(t, NC / 2) {
+      const uint32_t i = t * (kWave * 2) + lane * 2;
+      if (i < valid) {
+        const uint2 a = *reinterpret_cast<const uint2*>(pos_at(i));
+        Pack<int64_t, 2> pi;
+        pi.e[0] = index_of(i, a.x);
+        pi.e[1] = index_of(i + 1, a.y);
+        *reinterpret_cast<Pack<int64_t, 2>*>(oi + i) = pi;
+      }
+    } ATK_STATIC_END;
+  }
+}
+
 // Exact recomputation of one lane's V columns over sub-rows [p0, p1) (plus the
 // partial sub-row when `with_rem`), through order keys, one column at a time.
 // Off the hot path: kept small in registers rather than fast.
@@ -1328,7 +1429,12 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
   using word_t = typename MergeWord<E>::word_t;
   constexpr size_t kHandArea = (size_t)(W - 1) * Queue::kHandBytes;
   constexpr size_t kWordArea = (size_t)kTileCols * J * sizeof(word_t);
-  __shared__ __align__(16) unsigned char lds[kHandArea > kWordArea ? kHandArea : kWordArea];
+  // final results leave through LDS, in whole-wave stores of adjacent bytes
+  constexpr bool kTransposed = Transposed<E, J, V>::available;
+  constexpr size_t kOutArea = kTransposed ? Transposed<E, J, V>::kBytes : 0;
+  constexpr size_t kLdsArea = kHandArea > kWordArea ? (kHandArea > kOutArea ? kHandArea : kOutArea)
+                                                    : (kWordArea > kOutArea ? kWordArea : kOutArea);
+  __shared__ __align__(16) unsigned char lds[kLdsArea];
   if constexpr (W > 1) {
     // waves 1.. hand their queues to wave 0 through LDS
     if (wave > 0) queue.hand_over(lds + (size_t)(wave - 1) * Queue::kHandBytes, lane);
@@ -1355,7 +1461,11 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
     exact_columns<E, J, V>(xr, g, out, row, slab, col, s0, W > 1 ? s1 : p1, last_slab);
   } else {
     queue.fix_zeros(xr, g.b, col);
-    emit<E, J, V>(g, out, row, slab, col, queue);
+    if constexpr (kTransposed) {
+      if (out.part_values != nullptr) emit<E, J, V>(g, out, row, slab, col, queue);
+    } else {
+      emit<E, J, V>(g, out, row, slab, col, queue);
+    }
     if constexpr (E::key_bits <= 32) {
       if (ranges.range != nullptr) {
         low = ~0u; high = 0u;
@@ -1366,6 +1476,11 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
         } ATK_STATIC_END;
       }
     }
+  }
+  if constexpr (kTransposed) {
+    // (wave-uniform: whole waves get here, the lanes beyond the row's last column included)
+    if (g.fold == 1 && !redo && out.part_values == nullptr)
+      emit_transposed<E, J, V>(g, out, row, (int64_t)col_tile * kTileCols, lane, queue, lds);
   }
   if constexpr (E::key_bits <= 32) {
     if (ranges.range != nullptr) {
