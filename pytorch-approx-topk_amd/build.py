@@ -56,6 +56,17 @@ def build(force: bool = False, verbose: bool = True) -> str:
         r = subprocess.run(cmd, capture_output=True, text=True)
         return cmd, r
 
+    # the translation units with the most kernels first (the per-type instances of the streaming
+    # and the one-workgroup-per-row kernels take minutes each), so that none of them is left for the end
+    def weight(cmd):
+        name = os.path.basename(cmd[-3])
+        heavy = ("stage1_stream_f16", "stage1_stream_bf16", "stage1_stream_i16", "fused_row_f16", "fused_row_bf16",
+                 "fused_row_i16", "fused_row_", "stage1_stream_", "stage2_chain", "stage1_contig_")
+        for rank, prefix in enumerate(heavy):
+            if name.startswith(prefix):
+                return rank
+        return len(heavy)
+    jobs.sort(key=weight)
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         for cmd, r in ex.map(run, jobs):
             # hipcc's host pass warns that it does not know the packed-fp32 feature.

@@ -46,11 +46,18 @@ static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t row
 template <typename E, int J, int V, int MAXW, typename pos_t>
 static int launch_one(const Plan& pl, const typename E::raw_t* x, int64_t rows, const Geom& g, uint32_t k0,
                       uint32_t k, typename E::raw_t* values, IndexOut indices, hipStream_t stream) {
-  if constexpr (stream::PackedKey<E>::available && sizeof(typename E::raw_t) == 2 && sizeof(pos_t) == 2) {
-    // packed queues need every sub-row number to fit 16 bits, as pos_t == uint16_t does
-    if (pl.packed) return launch_packed<E, J, V, MAXW, pos_t, true>(pl, x, rows, g, k0, k, values, indices, stream);
+  constexpr int VF = stream::full_vec((int)sizeof(typename E::raw_t));
+  if constexpr (stream::PackedKey<E>::available && sizeof(typename E::raw_t) == 2 && V == VF / 2) {
+    // Half the load width is the packed queues' (and only theirs: the planner halves it for
+    // them alone); they need every sub-row number to fit 16 bits, as pos_t == uint16_t does.
+    if constexpr (sizeof(pos_t) == 2) {
+      if (pl.packed) return launch_packed<E, J, V, MAXW, pos_t, true>(pl, x, rows, g, k0, k, values, indices, stream);
+    }
+    return ATK_ERR_ARG;  // the planner never asks for it
+  } else {
+    if (pl.packed) return ATK_ERR_ARG;  // (packed queues at full load width: never planned)
+    return launch_packed<E, J, V, MAXW, pos_t, false>(pl, x, rows, g, k0, k, values, indices, stream);
   }
-  return launch_packed<E, J, V, MAXW, pos_t, false>(pl, x, rows, g, k0, k, values, indices, stream);
 }
 
 template <typename E, int J, int VF>

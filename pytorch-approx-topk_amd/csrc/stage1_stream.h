@@ -886,14 +886,19 @@ __device__ __forceinline__ void emit(const Geom& g, const Sink<typename E::raw_t
 // from the next lane's for the banks -- and read them back in the order of the
 // output.  `col0`: the tile's first column; lanes beyond the row's last column
 // hold nothing that is read.  One wave: its LDS accesses complete in program
-// order, so nothing waits on a barrier.
+// order, so nothing waits on a barrier.  The trip through LDS is a few hundred
+// cycles at the end of every workgroup, which a launch of few workgroups, or one
+// whose output is small beside its input, does not get back: fp16 [256, 65536]
+// k=4096 j=4 (512 workgroups) 14.2 -> 15.5 us; the planner decides (Plan::wave_stores).
 template <typename E, int J, int V>
 struct Transposed {
   using raw_t = typename E::raw_t;
   static constexpr int NC = V * J;                           // entries of a lane
   static constexpr int kPerStore = 16 / (int)sizeof(raw_t);  // elements in 16 bytes
-  // whole 16-byte pieces on both sides, elements of up to four bytes
-  static constexpr bool available = V > 1 && sizeof(raw_t) <= 4 && NC % 4 == 0 && NC % kPerStore == 0;
+  // whole 16-byte pieces on both sides, elements of up to four bytes; not for eight 4-byte
+  // entries a lane (fp32 [128, 2^20] k=65536 j=2: 108.6-109.6 us either way)
+  static constexpr bool available = V > 1 && sizeof(raw_t) <= 4 && NC % 4 == 0 && NC % kPerStore == 0 &&
+                                    (NC * 8 >= 128 || sizeof(raw_t) < 4) && J != 3;  // (j = 3: not built)
   static constexpr size_t kRawPitch = (size_t)NC * sizeof(raw_t) + 16;  // bytes from lane to lane
   static constexpr size_t kPosPitch = (size_t)NC * 4 + 16;
   static constexpr size_t kPosArea = kWave * kRawPitch;                 // where the sub-row numbers start
@@ -1391,8 +1396,11 @@ __device__ __forceinline__ void fold_columns_exact(const typename E::raw_t* __re
 // E: element traits; J: entries kept per bucket; V: columns per lane; W: waves
 // per workgroup, sharing one column tile and splitting its sub-rows; U: loads
 // kept in flight per lane; RUN: exact sub-rows per wave when known (else 0);
-// PACKED: packed 16-bit queues.
-template <typename E, int J, int V, int W, int U, int RUN, bool PACKED>
+// PACKED: packed 16-bit queues; WAVE_STORES: final results leave through LDS
+// (emit_transposed; a kernel of its own rather than a branch: with both ways
+// out in one kernel, fp16 [256, 2^20] k=4096 j=2 took 117 instead of 110 us the
+// usual way).
+template <typename E, int J, int V, int W, int U, int RUN, bool PACKED, bool WAVE_STORES = false>
 __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) void stream_kernel(
     const typename E::raw_t* __restrict__ x, const Sink<typename E::raw_t> out, const Geom g,
     const KeyRangeOut ranges) {
@@ -1430,7 +1438,8 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
   constexpr size_t kHandArea = (size_t)(W - 1) * Queue::kHandBytes;
   constexpr size_t kWordArea = (size_t)kTileCols * J * sizeof(word_t);
   // final results leave through LDS, in whole-wave stores of adjacent bytes
-  constexpr bool kTransposed = Transposed<E, J, V>::available;
+  constexpr bool kTransposed = WAVE_STORES;
+  static_assert(!WAVE_STORES || Transposed<E, J, V>::available, "see Transposed");
   constexpr size_t kOutArea = kTransposed ? Transposed<E, J, V>::kBytes : 0;
   constexpr size_t kLdsArea = kHandArea > kWordArea ? (kHandArea > kOutArea ? kHandArea : kOutArea)
                                                     : (kWordArea > kOutArea ? kWordArea : kOutArea);
@@ -1461,11 +1470,7 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
     exact_columns<E, J, V>(xr, g, out, row, slab, col, s0, W > 1 ? s1 : p1, last_slab);
   } else {
     queue.fix_zeros(xr, g.b, col);
-    if constexpr (kTransposed) {
-      if (out.part_values != nullptr) emit<E, J, V>(g, out, row, slab, col, queue);
-    } else {
-      emit<E, J, V>(g, out, row, slab, col, queue);
-    }
+    if constexpr (!kTransposed) emit<E, J, V>(g, out, row, slab, col, queue);
     if constexpr (E::key_bits <= 32) {
       if (ranges.range != nullptr) {
         low = ~0u; high = 0u;
@@ -1479,8 +1484,7 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
   }
   if constexpr (kTransposed) {
     // (wave-uniform: whole waves get here, the lanes beyond the row's last column included)
-    if (g.fold == 1 && !redo && out.part_values == nullptr)
-      emit_transposed<E, J, V>(g, out, row, (int64_t)col_tile * kTileCols, lane, queue, lds);
+    if (!redo) emit_transposed<E, J, V>(g, out, row, (int64_t)col_tile * kTileCols, lane, queue, lds);
   }
   if constexpr (E::key_bits <= 32) {
     if (ranges.range != nullptr) {
@@ -1613,6 +1617,7 @@ struct Plan {
   uint32_t full_rows, rem, pad_tail;  // of the scanned matrix
   uint32_t slabs, slab_len, col_tiles;
   bool merge;         // the merge kernel follows (several slabs)
+  bool wave_stores;   // final results leave through LDS in whole-wave stores
   size_t part_values_off, part_pos_off, ws_bytes;
 };
 

@@ -7,8 +7,9 @@
 namespace atk {
 namespace stream {
 
-template <typename E, int J, int V, int W, int RUN>
-static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
+// WS: results through LDS in whole-wave stores (Plan::wave_stores)
+template <typename E, int J, int V, int W, int RUN, bool WS>
+static int launch_out(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
                       const Geom& g, dim3 grid, hipStream_t stream, const KeyRangeOut& left) {
   constexpr int U = loads_in_flight(DtypeOf<E>::value, J, V, false);
   if constexpr (PackedKey<E>::available) {
@@ -16,23 +17,36 @@ static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typ
       constexpr int UP = loads_in_flight(DtypeOf<E>::value, J, V, true);
       if constexpr (deep_loads_for_short_columns(DtypeOf<E>::value, J, V, true, RUN, 0) && UP != 8) {
         if (deep_loads_for_short_columns(DtypeOf<E>::value, J, V, true, RUN, g.full_rows)) {
-          hipLaunchKernelGGL((stream_kernel<E, J, V, W, 8, RUN, true>), grid, dim3(kWave * W), 0, stream, x, out, g,
-                             left);
+          hipLaunchKernelGGL((stream_kernel<E, J, V, W, 8, RUN, true, WS>), grid, dim3(kWave * W), 0, stream, x, out,
+                             g, left);
           return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
         }
       }
-      hipLaunchKernelGGL((stream_kernel<E, J, V, W, UP, RUN, true>), grid, dim3(kWave * W), 0, stream, x, out, g, left);
+      hipLaunchKernelGGL((stream_kernel<E, J, V, W, UP, RUN, true, WS>), grid, dim3(kWave * W), 0, stream, x, out, g,
+                         left);
       return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
     }
   }
   // (the general queues hand over twice the bytes of the packed ones: combinations of theirs
   // beyond the LDS budget, which the planner never picks, are not compiled)
   if constexpr (merge_lds_bytes(V, J, W, (int)sizeof(typename Cmp<E>::cmp_t) + 4) <= merge_lds_limit(8)) {
-    hipLaunchKernelGGL((stream_kernel<E, J, V, W, U, RUN, false>), grid, dim3(kWave * W), 0, stream, x, out, g, left);
+    hipLaunchKernelGGL((stream_kernel<E, J, V, W, U, RUN, false, WS>), grid, dim3(kWave * W), 0, stream, x, out, g,
+                       left);
     return hipGetLastError() == hipSuccess ? ATK_OK : ATK_ERR_LAUNCH;
   } else {
     return ATK_ERR_ARG;
   }
+}
+
+template <typename E, int J, int V, int W, int RUN>
+static int launch_run(const Plan& pl, const typename E::raw_t* x, const Sink<typename E::raw_t>& out,
+                      const Geom& g, dim3 grid, hipStream_t stream, const KeyRangeOut& left) {
+  if constexpr (Transposed<E, J, V>::available) {
+    if (pl.wave_stores) return launch_out<E, J, V, W, RUN, true>(pl, x, out, g, grid, stream, left);
+  } else if (pl.wave_stores) {
+    return ATK_ERR_ARG;  // the planner never asks for it
+  }
+  return launch_out<E, J, V, W, RUN, false>(pl, x, out, g, grid, stream, left);
 }
 
 template <typename E, int J, int V, int W>

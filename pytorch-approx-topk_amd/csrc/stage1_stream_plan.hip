@@ -12,6 +12,8 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 constexpr int64_t kTargetWaves = 1024;
 // Sub-rows worth giving to one wave before a row is also cut into slabs.
 constexpr int64_t kSlabRun = 16;
+// Fewest workgroups of a launch whose results take the trip through LDS.
+constexpr int64_t kTransposeGroups = 2048;
 // Sub-rows a wave keeps when a row is cut only to put a second wave on every SIMD.
 constexpr int64_t kLongRun = 64;
 // Fewest sub-rows a wave scans when several share a tile: with runs of 2 the
@@ -132,6 +134,19 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int layout, int dtype
     pl.part_pos_off = align_up(entries * es, 256);
     pl.ws_bytes = pl.part_pos_off + align_up(entries * sizeof(uint32_t), 256);
   }
+  // Results through LDS in whole-wave stores (emit_transposed): when a lane's stretch of
+  // the output is long (its indices 128 bytes or more) or its elements short, the launch
+  // has workgroups by the thousand, and a workgroup writes at least an eighth of what it reads
+  // (at a twelfth, fp16 [256, 2^20] k=16384: j=2 112.6 -> 115.1 us, j=4 118.2 -> 115.2 us, j=1 104.9 -> 102.5 us).
+  pl.wave_stores = false;
+  if (pl.vec > 1 && es <= 4 && !pl.merge && pl.fold == 1) {
+    const int64_t entries = (int64_t)pl.vec * j;  // of a lane
+    const bool whole_pieces = entries % 4 == 0 && entries % (16 / es) == 0 && j != 3;  // (Transposed::available)
+    const int64_t groups = rows * (int64_t)pl.col_tiles;
+    const int64_t in_bytes = full * kWave * pl.vec * es, out_bytes = kWave * entries * (es + 8);
+    pl.wave_stores = whole_pieces && (entries * 8 >= 128 || es < 4) && groups >= kTransposeGroups &&
+                     out_bytes * 8 >= in_bytes;
+  }
   pl.ok = true;
   return pl;
 }
@@ -162,7 +177,8 @@ bool describe_stage1_stream(const void* x, int64_t rows, int64_t n, int64_t row_
          ", V=" + std::to_string(pl.vec) + ", W=" + std::to_string(pl.waves) + ", U=" + std::to_string(loads) +
          ", RUN=" + std::to_string(pl.run) + ", PACKED=" + (pl.packed ? "1" : "0") + "> grid=" +
          std::to_string(rows * (int64_t)pl.slabs * pl.col_tiles) + " block=" + std::to_string(64 * pl.waves) +
-         " fold=" + std::to_string(pl.fold) + " slabs=" + std::to_string(pl.slabs);
+         " fold=" + std::to_string(pl.fold) + " slabs=" + std::to_string(pl.slabs) +
+         (pl.wave_stores ? " wave-stores" : "");
   if (pl.merge) out += " + stream_merge_kernel<" + std::string(dtype_name(dtype)) + ", J=" + std::to_string(j) + ">";
   return true;
 }
