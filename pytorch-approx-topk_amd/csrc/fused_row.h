@@ -274,7 +274,11 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
 
 // Packed queues of up to 16 entries per lane are held to 64 vector registers
 // (eight waves per SIMD: four 8-wave workgroups per CU); what does not fit is
-// spilled where the pressure peaks, in the rarely taken LDS path.
+// spilled where the pressure peaks, in the rarely taken LDS path.  The scan of
+// contiguous buckets with 16 entries per lane is left its 80 registers (six
+// waves per SIMD): its loads of whole buckets spill in the scan itself
+// otherwise (fp16 [1024, 32768] k=2048 j=4 k_mult=4 36 -> 31 us, [4096, 8192]
+// k=512 45 -> 36 us; with 8 entries per lane the 64 registers win by a tenth).
 // CONTIG: the row's buckets are contiguous runs of g.full_rows elements of at
 // most 256 bytes (no remainder, whole tiles, one wave per tile).  The scan differs,
 // the way an index is put together, and which buckets a lane holds: V buckets
@@ -282,7 +286,7 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
 // of every lane's first bucket, then of every lane's second, ...
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED, bool CONTIG = false>
 __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80)))
-__attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 ? 8 : 1))) void fused_regs_kernel(
+__attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 8) ? 8 : 1))) void fused_regs_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
     const IndexOut indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t hand_off,
     uint32_t k0, uint32_t k, int index_bits, int staged) {
