@@ -1,10 +1,14 @@
 """Builds libapprox_topk_hip.so for gfx950 with hipcc, in-tree.
 
-    python pytorch-approx-topk_amd/build.py [--force]
+    python pytorch-approx-topk_amd/build.py [--force] [--trace]
 
 Every .hip file under csrc/ is compiled to an object (in parallel) and linked
 into approx_topk/libapprox_topk_hip.so, next to the Python package that loads
 it.  Nothing is linked against libtorch: the library speaks a C ABI only.
+
+--trace builds a second library, approx_topk/libapprox_topk_hip_trace.so, whose long
+kernels stamp a clock at their phase boundaries (csrc/atk_trace.h); it is what
+benchmarks/phase_timeline.py loads, and nothing else does.
 """
 from __future__ import annotations
 
@@ -37,18 +41,21 @@ def _newer(target: str, deps: list[str]) -> bool:
     return all(os.path.getmtime(d) <= t for d in deps)
 
 
-def build(force: bool = False, verbose: bool = True) -> str:
-    os.makedirs(OBJ, exist_ok=True)
+def build(force: bool = False, verbose: bool = True, trace: bool = False) -> str:
+    obj_dir, lib, flags = OBJ, LIB, list(FLAGS)
+    if trace:
+        obj_dir, lib, flags = OBJ + "_trace", LIB[:-3] + "_trace.so", flags + ["-DATK_TRACE"]
+    os.makedirs(obj_dir, exist_ok=True)
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     headers = sorted(glob.glob(os.path.join(CSRC, "*.h"))) + [
         os.path.join(os.path.dirname(HERE), "include", "approx_topk_hip.h")]
     jobs = []
     objects = []
     for src in sources:
-        obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+        obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
         objects.append(obj)
         if force or not _newer(obj, [src] + headers):
-            jobs.append([HIPCC, *FLAGS, "-c", src, "-o", obj])
+            jobs.append([HIPCC, *flags, "-c", src, "-o", obj])
 
     def run(cmd):
         if verbose:
@@ -75,12 +82,12 @@ def build(force: bool = False, verbose: bool = True) -> str:
                 raise RuntimeError(f"{' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
             if verbose and err.strip():
                 print(err, file=sys.stderr)
-    if force or jobs or not _newer(LIB, objects):
-        cmd, r = run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objects])
+    if force or jobs or not _newer(lib, objects):
+        cmd, r = run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objects])
         if r.returncode != 0:
             raise RuntimeError(f"{' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv))
+    print(build(force="--force" in sys.argv, trace="--trace" in sys.argv))

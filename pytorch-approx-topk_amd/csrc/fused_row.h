@@ -20,6 +20,7 @@
 
 #include "stage1_stream.h"
 #include "stage2_select.h"
+#include "atk_trace.h"
 
 namespace atk {
 namespace fused {
@@ -279,12 +280,15 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
 // waves per SIMD): its loads of whole buckets spill in the scan itself
 // otherwise (fp16 [1024, 32768] k=2048 j=4 k_mult=4 36 -> 31 us, [4096, 8192]
 // k=512 45 -> 36 us; with 8 entries per lane the 64 registers win by a tenth).
+// PAST_CACHE: staged results leave four per thread (staged == 2) in non-temporal stores; a
+// kernel of its own, because as a branch it cost the usual way out 2 us of 36 (fp16 [4096, 8192]
+// k=512 j=4 k_mult=4) through the registers it moved.
 // CONTIG: the row's buckets are contiguous runs of g.full_rows elements of at
 // most 256 bytes (no remainder, whole tiles, one wave per tile).  The scan differs,
 // the way an index is put together, and which buckets a lane holds: V buckets
 // kWave apart (bucket_of), so that a wave's candidates in their order are those
 // of every lane's first bucket, then of every lane's second, ...
-template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED, bool CONTIG = false>
+template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED, bool CONTIG = false, bool PAST_CACHE = false>
 __global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80)))
 __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 8) ? 8 : 1))) void fused_regs_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
@@ -317,6 +321,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
   const int64_t row = blockIdx.x;
   const raw_t* xr = x + row * g.row_stride;
 
+  ATK_TRACE_GROUP(0);
   const uint32_t part = wave % split;   // which share of the sub-rows
   const uint32_t tile = wave / split;   // every tile has its waves: tiles * split == waves
   const uint32_t p0 = __builtin_amdgcn_readfirstlane((uint32_t)(((uint64_t)g.full_rows * part) / split));
@@ -355,10 +360,12 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
     // with the hand-over area, which may lie in the same place.
     if (split > 1) __syncthreads();
   }
+  ATK_TRACE_GROUP(1);
   for (uint32_t i = tid * 4; i < 2 * regs::kHistWords; i += nt * 4)
     *reinterpret_cast<uint4*>(&hist[i]) = make_uint4(0, 0, 0, 0);
   if (tid == 0) rs.list_count = 0;
   const bool nan_row = __syncthreads_or(any_nan);
+  ATK_TRACE_GROUP(2);
 
   // (keys are taken from the queues where they are used rather than kept: registers)
   // (Packed entries carry the sub-row number below the key, which is the order of the
@@ -420,6 +427,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
           *reinterpret_cast<uint4*>(&other[i]) = make_uint4(0, 0, 0, 0);
       }
       __syncthreads();
+      ATK_TRACE_GROUP(pass == 0 ? 3 : 4);
       prefix |= (sel_t)rs.digit << shift;
       mask |= (sel_t)dmask << shift;
       need = rs.need;
@@ -507,6 +515,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
     }
   }
 
+  ATK_TRACE_GROUP(5);
   // survivors among this lane's candidates
   uint32_t selected = 0;  // bit e: candidate e survives
   ATK_STATIC_FOR(e, NC) {
@@ -531,6 +540,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
     if (lane == kWave - 1) rs.wave_total[wave] = before;
   }
   __syncthreads();
+  ATK_TRACE_GROUP(6);
   {
     uint32_t waves_before = 0;
     for (uint32_t w = 0; w < wave; ++w) waves_before += rs.wave_total[w];
@@ -553,6 +563,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
         o += (selected >> e) & 1u;
       } ATK_STATIC_END;
       __syncthreads();
+      ATK_TRACE_GROUP(7);
       auto result = [&](uint2 w, raw_t& value) __attribute__((always_inline)) -> uint32_t {
         const typename Queue::Unstaged u = queue.unstage(w);
         const uint32_t index = CONTIG ? u.column * g.full_rows + u.sub_row : u.sub_row * (uint32_t)g.b + u.column;
@@ -570,6 +581,36 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
           index[1] = result(make_uint2(e01.z, e01.w), pv.e[1]);
           index[2] = result(make_uint2(e23.x, e23.y), pv.e[2]);
           index[3] = result(make_uint2(e23.z, e23.w), pv.e[3]);
+          if constexpr (PAST_CACHE) {
+            // (non-temporal stores: one round of workgroups with a sizeable output, see the planner)
+            typedef uint32_t nt4 __attribute__((ext_vector_type(4)));
+            typedef uint32_t nt2 __attribute__((ext_vector_type(2)));
+            if (values != nullptr) {
+              if constexpr (sizeof(raw_t) == 4) {
+                nt4 w;
+                __builtin_memcpy(&w, &pv, 16);
+                __builtin_nontemporal_store(w, reinterpret_cast<nt4*>(ov + at));
+              } else if constexpr (sizeof(raw_t) == 2) {
+                nt2 w;
+                __builtin_memcpy(&w, &pv, 8);
+                __builtin_nontemporal_store(w, reinterpret_cast<nt2*>(ov + at));
+              } else {
+                uint32_t w;
+                __builtin_memcpy(&w, &pv, 4);
+                __builtin_nontemporal_store(w, reinterpret_cast<uint32_t*>(ov + at));
+              }
+            }
+            if (indices.narrow) {
+              const nt4 w = {index[0], index[1], index[2], index[3]};
+              __builtin_nontemporal_store(w, reinterpret_cast<nt4*>(static_cast<int32_t*>(indices.base) + oi + at));
+            } else {
+              nt4* out = reinterpret_cast<nt4*>(static_cast<int64_t*>(indices.base) + oi + at);
+              const nt4 lo = {index[0], 0u, index[1], 0u}, hi = {index[2], 0u, index[3], 0u};
+              __builtin_nontemporal_store(lo, out);
+              __builtin_nontemporal_store(hi, out + 1);
+            }
+            continue;
+          }
           if (values != nullptr) *reinterpret_cast<stream::Pack<raw_t, 4>*>(ov + at) = pv;
           if (indices.narrow) {
             stream::Pack<int32_t, 4> pi;
@@ -593,6 +634,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
           indices.put(oi + at, (int64_t)index);
         }
       }
+      ATK_TRACE_GROUP(8);
       return;
     }
   }
@@ -630,6 +672,7 @@ struct Plan {
   bool contig;          // contiguous buckets of a few elements each (in_registers only)
   bool in_registers;    // all tiles are scanned at once: the candidates stay in registers through stage 2
   bool staged;          // in_registers: the survivors are gathered in LDS and leave in whole-wave stores
+  bool past_cache;      // staged: ... in non-temporal stores (one round of workgroups with a sizeable output)
 };
 
 Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout, int dtype, bool aligned);

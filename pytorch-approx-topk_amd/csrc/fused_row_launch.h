@@ -13,20 +13,27 @@ static int launch_packed(const Plan& pl, const typename E::raw_t* x, int64_t row
     if (pl.in_registers) return ATK_ERR_ARG;  // (the register kernel is built for eight waves)
   } else if (pl.in_registers) {
     auto kern = fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED>;
+    // staged results leave four per thread when the outputs allow 16-byte stores, and then,
+    // when the planner says so, past the cache
+    const bool wide = k % 4 == 0 && (uintptr_t)values % 16 == 0 && (uintptr_t)indices.base % 16 == 0;
+    [[maybe_unused]] const bool past_cache = pl.staged && pl.past_cache && wide;
     // contiguous short buckets: 16-bit positions, elements of two (packed queues) or four bytes
     constexpr int ES = (int)sizeof(typename E::raw_t);
     if constexpr (sizeof(pos_t) == 2 && ((ES == 2 && PACKED) || ES == 4) && V == 4) {
-      if (pl.contig) kern = fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED, true>;
+      if (pl.contig)
+        kern = past_cache ? fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED, true, true>
+                          : fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED, true>;
     } else if (pl.contig) {
       return ATK_ERR_ARG;  // the planner never asks for it
+    }
+    if constexpr (sizeof(pos_t) == 2 && ES <= 4) {  // (what staging asks for)
+      if (!pl.contig && past_cache) kern = fused_regs_kernel<E, J, V, MAXW, pos_t, PACKED, false, true>;
     }
     if (pl.lds_bytes > 48 * 1024) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)pl.lds_bytes) != hipSuccess)
         return ATK_ERR_LAUNCH;
     }
-    // staged results leave four per thread when the outputs allow 16-byte stores
-    const bool wide = k % 4 == 0 && (uintptr_t)values % 16 == 0 && (uintptr_t)indices.base % 16 == 0;
     const int staged = pl.staged ? (wide ? 2 : 1) : 0;
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(kWave * pl.waves), pl.lds_bytes, stream, x, values,
                        indices, g, pl.tiles, pl.split, pl.hand_off, k0, k, pl.index_bits, staged);

@@ -34,6 +34,21 @@ constexpr int64_t kShortBucket = 256;
 constexpr size_t kShortRow = 128 * 1024, kLongRow = 512 * 1024;
 }  // namespace
 
+// Staged results leave in non-temporal stores when the launch is one round of workgroups
+// (no more rows than the GPU holds at once) and a row's results are an eighth of its bytes
+// or more.  What a kernel has written sits in the L2 of its XCD until the kernel ends and
+// is written back then, with nothing left to hide it behind: first workgroup's start to
+// last store 22.8 us of fp16 [1024, 32768] k=2048 j=4 k_mult=4's 27.1 us per call.  Sent
+// past the cache the results travel while other workgroups still work: 27.6 -> 25.4 us
+// there, fp16 [256, 131072] k=4096 j=4 k_mult=2 22.2 -> 20.1 us, fp32 [512, 32768] k=2048
+// j=4 k_mult=4 24.4 -> 23.1 us.  With several rounds the write-back hides behind the
+// later rounds by itself and the stores past the cache cost more than they save ([4096,
+// 8192] k=512 35.6 -> 36.9 us, [2048, 32768] 46.3 -> 47.3 us), as they do with little
+// output ([1024, 65536] k=512 44.0 -> 45.1 us).
+static bool stores_past_cache(int64_t rows, int64_t n, int64_t k, int64_t es) {
+  return rows <= kManyRows && k * (es + 8) * 8 >= n * es;
+}
+
 // Contiguous buckets, all of one length of 16 to kShortBucket bytes, elements of
 // two or four bytes: a lane of the register kernel loads its four buckets whole.  The
 // alternative is a stage-1 kernel that copies spans of buckets through LDS and
@@ -74,6 +89,7 @@ static Plan plan_short_buckets(int64_t rows, int64_t n, int64_t k0, int j, int64
   pl.lds_bytes = cand_bytes > regs::kLdsBytes ? cand_bytes : regs::kLdsBytes;
   pl.staged = (size_t)k * 8 <= kLdsBudget;
   if (pl.staged && pl.lds_bytes < (size_t)k * 8) pl.lds_bytes = (size_t)k * 8;
+  pl.past_cache = pl.staged && stores_past_cache(rows, n, k, es);
   pl.ok = true;
   return pl;
 }
@@ -189,6 +205,7 @@ Plan make_plan(int64_t rows, int64_t n, int64_t k0, int j, int64_t k, int layout
   // survivors staged in LDS, eight bytes each (element, 32-bit index), when that fits
   pl.staged = pl.in_registers && pl.pos16 && es <= 4 && (size_t)k * 8 <= kLdsBudget;
   if (pl.staged && pl.lds_bytes < (size_t)k * 8) pl.lds_bytes = (size_t)k * 8;
+  pl.past_cache = pl.staged && stores_past_cache(rows, n, k, es);
   pl.ok = true;
   return pl;
 }
@@ -218,7 +235,7 @@ bool describe_fused_row(const void* x, int64_t rows, int64_t n, int64_t row_stri
          std::to_string(j) + ", V=" + std::to_string(pl.vec) + ", pos" + (pl.pos16 ? "16" : "32") +
          ", PACKED=" + (pl.packed ? "1" : "0") + "> grid=" + std::to_string(rows) + " block=" +
          std::to_string(64 * pl.waves) + " tiles=" + std::to_string(pl.tiles) + " split=" + std::to_string(pl.split) +
-         " lds=" + std::to_string(pl.lds_bytes) + (pl.in_registers && pl.staged ? " staged" : "") +
+         " lds=" + std::to_string(pl.lds_bytes) + (pl.in_registers && pl.staged ? (pl.past_cache ? " staged past-cache" : " staged") : "") +
          (pl.contig ? " short contiguous buckets" : "");
   return true;
 }

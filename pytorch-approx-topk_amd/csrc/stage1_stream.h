@@ -45,6 +45,7 @@
 
 #include "atk_device.h"
 #include "atk_launch.h"
+#include "atk_trace.h"
 #include "stage2_select.h"
 
 namespace atk {
@@ -1430,7 +1431,9 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
 
   const raw_t* xr = x + row * g.row_stride;
   Queue queue;
+  ATK_TRACE_WAVE((int)wave * 2);  // slots 2w, 2w + 1: wave w's scan; 16: the workgroup's end
   scan_run<E, J, V, U, RUN>(xr, g, col, live, p0, p1, last_slab && wave == W - 1, queue);
+  ATK_TRACE_WAVE((int)wave * 2 + 1);
 
   bool redo = queue.poisoned();
   // LDS: the hand-over area of waves 1.., later the merge words of a folded row
@@ -1502,6 +1505,7 @@ __global__ __launch_bounds__(kWave * W) __attribute__((amdgpu_waves_per_eu(4))) 
       if (block == 0 && lane < ranges.state_words) ranges.state[(size_t)row * ranges.state_words + lane] = 0;
     }
   }
+  ATK_TRACE_WAVE(16);
 }
 
 // Folds the slabs' partial queues of every bucket into the final result under

@@ -6,3 +6,5 @@ namespace stream {
 ATK_INSTANTIATE_STREAM(ATK_F16)
 }  // namespace stream
 }  // namespace atk
+
+ATK_TRACE_READER(atk_trace_stage1_stream_f16)  // (nothing, unless the library is built for the phase timelines)

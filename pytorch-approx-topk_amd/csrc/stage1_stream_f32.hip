@@ -6,3 +6,5 @@ namespace stream {
 ATK_INSTANTIATE_STREAM(ATK_F32)
 }  // namespace stream
 }  // namespace atk
+
+ATK_TRACE_READER(atk_trace_stage1_stream_f32)  // (nothing, unless the library is built for the phase timelines)

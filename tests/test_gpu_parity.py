@@ -309,6 +309,43 @@ def test_fused_rows_with_candidates_beyond_64_kib_of_lds(dtype, rows, n, k, j, k
     _check(x, k, -1, j=j, k_mult=k_mult)
 
 
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.int16, torch.float32, torch.int32])
+def test_fused_rows_results_past_the_cache(dtype, interleaved):
+    """One round of workgroups whose results are an eighth of the row or more: the kernel whose staged
+    results leave in non-temporal stores; with more rows, or misaligned outputs, the usual one.  The
+    same results either way, with int64 and int32 indices and with the indices alone."""
+    from approx_topk import _native
+    from approx_topk.experimental.compact_indices import topk as topk_int32, topk_indices
+    layout = _native.INTERLEAVED if interleaved else _native.BALANCED
+    n, k, j, k_mult = 8192, 512, 4, 4
+    g = torch.Generator().manual_seed(n + int(interleaved))
+    for rows, past in [(300, True), (1200, False)]:
+        x = torch.randint(-2000, 2000, (rows, n), generator=g)
+        x = (x / 16).to(dtype) if dtype.is_floating_point else x.to(dtype)
+        xg = x.cuda()
+        plan = _native.describe(xg, k * k_mult, j, k, layout)
+        assert ("past-cache" in plan) == past and "fused_regs_kernel" in plan, plan
+        _check(x, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+        ev, ei = oracle_topk(x, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+        v32, i32 = topk_int32(xg, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+        assert_same(v32, i32.long(), ev, ei, "int32 indices")
+        only = topk_indices(xg, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+        assert torch.equal(only.cpu().long(), ei)
+    # outputs that are not 16-byte aligned: single stores, not past the cache
+    values = torch.empty(300 * k + 1, dtype=dtype, device="cuda")[1:].view(300, k)
+    indices = torch.empty(300 * k + 1, dtype=torch.int64, device="cuda")[1:].view(300, k)
+    x = torch.randint(-2000, 2000, (300, n), generator=g)
+    x = (x / 16).to(dtype) if dtype.is_floating_point else x.to(dtype)
+    xg = x.cuda()
+    rc = _native.lib().atk_topk(xg.data_ptr(), 300, n, n, k * k_mult, j, k, layout, _native.dtype_code(dtype),
+                                values.data_ptr(), indices.data_ptr(), 0, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0  # (no workspace: both stages run in one kernel)
+    torch.cuda.synchronize()
+    ev, ei = oracle_topk(x, k, -1, j=j, k_mult=k_mult, interleaved=interleaved)
+    assert_same(values, indices, ev, ei, "misaligned outputs")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
 def test_fused_rows_special_values(dtype):
     g = torch.Generator().manual_seed(5)

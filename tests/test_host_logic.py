@@ -23,6 +23,8 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(handle, name), name
     assert set(_native._SIGNATURES) == declared
+    # the clock stamps of the phase timelines (csrc/atk_trace.h) exist only in a library built for them
+    assert not hasattr(handle, "atk_trace_fused_row_f16") and not hasattr(handle, "atk_trace_stage1_stream_f32")
     assert _native.lib().atk_version() == _native.ABI_VERSION
     assert _native.lib().atk_strerror(0) == b"ok"
     assert b"j must" in _native.lib().atk_strerror(-2)
