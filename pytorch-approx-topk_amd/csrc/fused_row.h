@@ -339,12 +339,36 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
   // packed entries: sub-row numbers 0..full_rows at the top of the low half, so
   // that the bits in which entries differ are the leading ones
   queue.set_position_shift(sizeof(pos_t) == 2 ? (uint32_t)__builtin_clz(g.full_rows | 1u) - 16u : 0u);
+  // The first radix pass over sel_key (below) takes its leading `bits0` bits.  With a wave per
+  // tile (split == 1) nothing else uses the LDS while the row is scanned, so the histograms are
+  // cleared before the scan and a wave counts its candidates' digits as soon as its own scan is
+  // done, rather than after the workgroup's slowest wave: one barrier phase less in the chain that
+  // every workgroup goes through after its scan.
+  constexpr bool kKeyHalf = CONTIG && PACKED;
+  const int shift_end = kKeyHalf ? 16 : queue.sel_constant_bits();
+  const int bits0 = Queue::sel_bits - shift_end < regs::kDigitBits ? Queue::sel_bits - shift_end : regs::kDigitBits;
+  const bool early = (CONTIG || split == 1) && k != k0 && k0 > regs::kListMax && bits0 > 0;
+  if (early) {
+    for (uint32_t i = tid * 4; i < 2 * regs::kHistWords; i += nt * 4)
+      *reinterpret_cast<uint4*>(&hist[i]) = make_uint4(0, 0, 0, 0);
+    if (tid == 0) rs.list_count = 0;
+    __syncthreads();
+  }
   bool any_nan = false;
   if (has_tile) {
     if constexpr (CONTIG) scan_short_buckets<E, J, V, PACKED, !PACKED>(xr, g.full_rows, col, queue);
     else if (split > 1) stream::scan_windows<E, J, V, U>(xr, g, col, live, part, split, part == split - 1, queue);
     else stream::scan_run<E, J, V, U, 0>(xr, g, col, live, p0, p1, true, queue);
     any_nan = queue.poisoned();
+  }
+  if (early && mine) {  // (a wave that met a NaN counts keys that mean nothing: the row leaves the fast path anyway)
+    const int shift0 = Queue::sel_bits - bits0;
+    const uint32_t dmask0 = (1u << bits0) - 1u;
+    ATK_STATIC_FOR(e, NC) {
+      sel_t key = queue.template sel_key<e / J, e % J>();
+      if constexpr (kKeyHalf) key &= (sel_t)0xffff0000u;
+      atomicAdd(&hist[regs::hist_slot((uint32_t)(key >> shift0) & dmask0)], 1u);
+    } ATK_STATIC_END;
   }
   if constexpr (!CONTIG) {
     if (split > 1) {
@@ -361,16 +385,17 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
     if (split > 1) __syncthreads();
   }
   ATK_TRACE_GROUP(1);
-  for (uint32_t i = tid * 4; i < 2 * regs::kHistWords; i += nt * 4)
-    *reinterpret_cast<uint4*>(&hist[i]) = make_uint4(0, 0, 0, 0);
-  if (tid == 0) rs.list_count = 0;
+  if (!early) {
+    for (uint32_t i = tid * 4; i < 2 * regs::kHistWords; i += nt * 4)
+      *reinterpret_cast<uint4*>(&hist[i]) = make_uint4(0, 0, 0, 0);
+    if (tid == 0) rs.list_count = 0;
+  }
   const bool nan_row = __syncthreads_or(any_nan);
   ATK_TRACE_GROUP(2);
 
   // (keys are taken from the queues where they are used rather than kept: registers)
   // (Packed entries carry the sub-row number below the key, which is the order of the
   // indices of equal keys in the interleaved layout only: sub-row first, then column.)
-  constexpr bool kKeyHalf = CONTIG && PACKED;
   auto key_of = [&](auto e_c) __attribute__((always_inline)) -> sel_t {
     constexpr int e = decltype(e_c)::value;
     if constexpr (kKeyHalf) return queue.template sel_key<e / J, e % J>() & (sel_t)0xffff0000u;
@@ -394,7 +419,6 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
   enum { kByPrefix, kByList, kGiveUp } how = kGiveUp;
   if (!nan_row) {
     int shift = Queue::sel_bits;
-    const int shift_end = kKeyHalf ? 16 : queue.sel_constant_bits();
     for (uint32_t pass = 0;; ++pass) {
       if (need == count) { how = kByPrefix; break; }
       if (count <= regs::kListMax) { how = kByList; break; }
@@ -403,20 +427,24 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
       shift -= bits;
       const uint32_t dmask = (1u << bits) - 1u;
       uint32_t* h = hist + (pass & 1u) * regs::kHistWords;
-      if (mine) {
-        if (pass == 0) {  // every candidate counts
-          ATK_STATIC_FOR(e, NC) {
-            const sel_t key = key_of(std::integral_constant<int, e>{});
-            atomicAdd(&h[regs::hist_slot((uint32_t)(key >> shift) & dmask)], 1u);
-          } ATK_STATIC_END;
-        } else {
-          ATK_STATIC_FOR(e, NC) {
-            const sel_t key = key_of(std::integral_constant<int, e>{});
-            if ((key & mask) == prefix) atomicAdd(&h[regs::hist_slot((uint32_t)(key >> shift) & dmask)], 1u);
-          } ATK_STATIC_END;
+      if (pass == 0 && early) {
+        // counted already, and the barrier that told of NaNs has published the counts
+      } else {
+        if (mine) {
+          if (pass == 0) {  // every candidate counts
+            ATK_STATIC_FOR(e, NC) {
+              const sel_t key = key_of(std::integral_constant<int, e>{});
+              atomicAdd(&h[regs::hist_slot((uint32_t)(key >> shift) & dmask)], 1u);
+            } ATK_STATIC_END;
+          } else {
+            ATK_STATIC_FOR(e, NC) {
+              const sel_t key = key_of(std::integral_constant<int, e>{});
+              if ((key & mask) == prefix) atomicAdd(&h[regs::hist_slot((uint32_t)(key >> shift) & dmask)], 1u);
+            } ATK_STATIC_END;
+          }
         }
+        __syncthreads();
       }
-      __syncthreads();
       if (wave == 0) {
         const regs::Found f = regs::find_bin_wave(h, need, count, lane);
         if (lane == 0) { rs.digit = f.digit; rs.need = f.need; rs.count = f.count; }
