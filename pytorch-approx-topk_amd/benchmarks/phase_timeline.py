@@ -3,10 +3,11 @@ library built with `python pytorch-approx-topk_amd/build.py --trace` (csrc/atk_t
 
     python pytorch-approx-topk_amd/benchmarks/phase_timeline.py fused  float16:1024:32768:2048:4:4
     python pytorch-approx-topk_amd/benchmarks/phase_timeline.py stream float32:1:67108864:16384:4:2
+    python pytorch-approx-topk_amd/benchmarks/phase_timeline.py solo   float32:1:67108864:16384:4:2
 
 A shape is dtype:rows:n:k:j:k_mult.  `fused` reads the stamps of fused_regs_kernel (both stages
 in one kernel), `stream` those of stream_kernel (stage 1; every wave's scan and the workgroup's
-end).  The call is repeated back to back and the stamps are those of the last launch; times are
+end), `solo` those of chain_solo_kernel (stage 2 of few rows of up to 32768 candidates in one launch).  The call is repeated back to back and the stamps are those of the last launch; times are
 microseconds since the first workgroup's start (the 100 MHz clock that every compute unit reads
 alike), as minimum / median / maximum over the workgroups, then by XCD (workgroup number mod 8).
 The stamps cost the kernel a little: its duration here is 1-3 % above the product library's.
@@ -30,6 +31,8 @@ from approx_topk import _native, topk  # noqa: E402
 
 SLOTS, GROUPS = 20, 16384  # csrc/atk_trace.h
 SHORT = {"float16": "f16", "float32": "f32"}
+SOLO_PHASES = ["start", "keys in registers, the digit's place known", "histogram counted", "cut digit found",
+               "members of the cut digit listed", "list ranked, earlier survivors counted", "written"]
 FUSED_PHASES = ["start", "first wave's scan done", "all waves done, histograms cleared", "first radix pass",
                 "last of the later passes", "cut known", "survivors placed", "survivors staged", "written"]
 
@@ -40,7 +43,7 @@ def three(a):
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("kernel", choices=["fused", "stream"])
+    ap.add_argument("kernel", choices=["fused", "stream", "solo"])
     ap.add_argument("shape")
     ap.add_argument("--calls", type=int, default=40, help="back-to-back calls before the stamps are read")
     ap.add_argument("--contiguous", action="store_true")
@@ -52,7 +55,8 @@ def main():
     kw = dict(j=j, k_mult=k_mult, interleaved=not args.contiguous)
     plan = _native.describe(xs[0], k * k_mult, j, k, _native.INTERLEAVED if not args.contiguous else _native.BALANCED)
     print(plan)
-    unit = ("fused_row_" if args.kernel == "fused" else "stage1_stream_") + SHORT[f[0]]
+    unit = {"fused": "fused_row_" + SHORT[f[0]], "stream": "stage1_stream_" + SHORT[f[0]],
+            "solo": "stage2_chain_select"}[args.kernel]
     reader = getattr(_native.lib(), "atk_trace_" + unit)
     reader.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
     for s in range(args.calls):
@@ -84,6 +88,13 @@ def main():
         scan = t[:, 1] - t0
         print("deciles of scan done:", np.round(np.sort(scan)[:: max(1, groups // 10)], 1))
         print("deciles of written:  ", np.round(np.sort(end)[:: max(1, groups // 10)], 1))
+    elif args.kernel == "solo":
+        groups = int(plan.split("chain_solo_kernel")[1].split("grid=")[1].split()[0])
+        t = t[:groups]
+        t0 = t[:, 0].min()
+        print("%-44s %7s %7s %7s" % ("us since the first workgroup's start", "min", "median", "max"))
+        for i, name in enumerate(SOLO_PHASES):
+            print("%-44s %s" % (name, three(t[:, i] - t0)))
     else:
         grid = int(plan.split("grid=")[1].split()[0])
         waves = int(plan.split("block=")[1].split()[0]) // 64

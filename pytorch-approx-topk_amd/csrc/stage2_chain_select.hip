@@ -38,6 +38,7 @@
 // one-workgroup kernel: same survivors, same order.
 #include "atk_device.h"
 #include "atk_launch.h"
+#include "atk_trace.h"
 #include "stage2_select.h"
 
 namespace atk {
@@ -485,6 +486,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   const raw_t* cv = cand_values + (int64_t)row * k0;
   const int64_t* ci = cand_indices + (int64_t)row * k0;
 
+  ATK_TRACE_GROUP(0);
   // (the key ranges are asked for first, so that they travel with the keys; OWN_RANGE:
   // stage 1 left none, and the range is that of the keys read below)
   uint2 folded = make_uint2(~0u, 0u);
@@ -515,15 +517,18 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   }
   uint32_t low, shift;
   regs::digit_from_folded<kSoloThreads>(folded, red, low, shift);  // (its barrier covers the clearing)
+  ATK_TRACE_GROUP(1);
 #pragma unroll
   for (int u = 0; u < NPT; ++u)
     if (valid(u)) atomicAdd(&hist[(key[u] - low) >> shift], 1u);
   __syncthreads();
+  ATK_TRACE_GROUP(2);
   if (wave == 0) {
     const regs::Found f = regs::find_bin_wave<false>(hist, k, k0, lane);
     if (lane == 0) found = f;
   }
   __syncthreads();
+  ATK_TRACE_GROUP(3);
   regs::Found f = found;
   // The cut digit holds more candidates than the list: they are counted again by
   // the next bits of their offsets, which narrows the digit, until its members
@@ -781,6 +786,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     ats[n + tid] = ~0u;
   }
   __syncthreads();
+  ATK_TRACE_GROUP(4);
   // This thread's own candidate, asked for together with the listed members'
   // indices: one trip to memory for both.  (Asked for with the keys at the top,
   // the index load made the kernel 5 us slower, measured.)
@@ -813,6 +819,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     }
     for (uint32_t i = tid; i < n; i += kSoloThreads) before += (ats[i] < g * kSoloThreads && words[i] >= cut) ? 1u : 0u;
   }
+  ATK_TRACE_GROUP(5);
   // this thread's own candidate
   const uint32_t own_d = (own_key - low) >> shift;
   const bool sel = own_valid && (own_d > f.digit ||
@@ -835,6 +842,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
       indices.put((int64_t)row * k + at, (int64_t)(uint32_t)~own_inv);
     }
   }
+  ATK_TRACE_GROUP(6);
 }
 
 // Rows the one-launch form takes: short enough for the keys to sit in registers,
@@ -1028,3 +1036,5 @@ int launch_chain_select(const void* cand_values, const int64_t* cand_indices, in
 }
 
 }  // namespace atk
+
+ATK_TRACE_READER(atk_trace_stage2_chain_select)  // (nothing, unless the library is built for the phase timelines)
