@@ -492,7 +492,7 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
     // entry t and counts the better ones): the need-th best is the cut.  An entry
     // is one 64-bit word when key and index fit 32 bits each (key above inverted
     // index: a larger word is a better candidate), else two.  The list is read
-    // eight entries at a time; its last group is filled up with entries that
+    // four entries at a time; its last group is filled up with entries that
     // beat nothing.
     constexpr bool kOneWord = sizeof(sel_t) == 4 && sizeof(idx_t) == 4;
     if (tid < 8u) {
@@ -520,12 +520,18 @@ __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 
       const uint64_t my_key = list_key[t];
       const uint64_t my_index = kOneWord ? 0ull : list_index[t];
       uint32_t better = 0;
-      for (uint32_t m = 0; m < count; m += 8) {
-        uint64_t key[8], index[8];
+      // (four entries per trip and no unrolling: with eight, the sixteen registers of a trip were
+      // what made the compiler spill part of the lane's candidates to scratch memory in the
+      // kernels held to 64 registers -- 9 to 24 registers, 13 to 35 MB of HBM traffic per launch
+      // of fp16 [1024, 32768] k=2048 j=4 k_mult=4, which takes 24.2 us without them against 25.9)
+      constexpr int kGroup = 4;
+#pragma nounroll
+      for (uint32_t m = 0; m < count; m += kGroup) {
+        uint64_t key[kGroup], index[kGroup];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) { key[u] = list_key[m + u]; index[u] = kOneWord ? 0ull : list_index[m + u]; }
+        for (int u = 0; u < kGroup; ++u) { key[u] = list_key[m + u]; index[u] = kOneWord ? 0ull : list_index[m + u]; }
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
+        for (int u = 0; u < kGroup; ++u)
           better += (key[u] > my_key || (!kOneWord && key[u] == my_key && index[u] < my_index)) ? 1u : 0u;
       }
       if (lane < count && better + 1 == need) {  // one lane
