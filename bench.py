@@ -34,7 +34,7 @@ MEASURED_TRAFFIC_BYTES = {
     "stream_kernel<f32, J=2, V=4, W=8, U=8, RUN=4, PACKED=0> grid=16384 block=512 fold=1 slabs=1": 637_658_986,
     # profiles/hbm_traffic_c1_c3_c4_c5.md (C5: the sum of its three kernels)
     "stream_kernel<f32, J=1, V=4, W=8, U=8, RUN=8, PACKED=0> grid=16 block=512 fold=1 slabs=1": 1_209_344,
-    "fused_regs_kernel<f16, J=4, V=4, pos16, PACKED=1> grid=1024 block=512 tiles=8 split=1 lds=32768 staged past-cache": 101060244,
+    "fused_regs_kernel<f16, J=4, V=4, pos16, PACKED=1> grid=1024 block=512 tiles=8 split=1 lds=32768 staged past-cache": 88597838,
     "fused_regs_kernel<f32, J=1, V=4, pos16, PACKED=0> grid=256 block=512 tiles=2 split=4 lds=19584 staged": 134_724_608,
     "stream_kernel<f32, J=4, V=4, W=4, U=8, RUN=0, PACKED=0> grid=256 block=256 fold=1 slabs=8 + "
     "stream_merge_kernel<f32, J=4> + chain_solo_kernel<f32> grid=32 block=1024": 275_389_132,
