@@ -280,6 +280,10 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
 // waves per SIMD): its loads of whole buckets spill in the scan itself
 // otherwise (fp16 [1024, 32768] k=2048 j=4 k_mult=4 36 -> 31 us, [4096, 8192]
 // k=512 45 -> 36 us; with 8 entries per lane the 64 registers win by a tenth).
+// (No cap on the scalar registers here: the packed kernels' eight waves per SIMD already hold the
+// compiler to 96, and the others, which cannot reach eight waves for their vector registers, spilled
+// 46-107 scalar registers into vector lanes under a cap of 80: fp32 [256, 131072] k=64 j=1 k_mult=8
+// 28.3 -> 28.0 us without it.)
 // PAST_CACHE: staged results leave four per thread (staged == 2) in non-temporal stores; a
 // kernel of its own, because as a branch it cost the usual way out 2 us of 36 (fp16 [4096, 8192]
 // k=512 j=4 k_mult=4) through the registers it moved.
@@ -289,7 +293,7 @@ __device__ __forceinline__ void scan_short_buckets(const typename E::raw_t* __re
 // kWave apart (bucket_of), so that a wave's candidates in their order are those
 // of every lane's first bucket, then of every lane's second, ...
 template <typename E, int J, int V, int MAXW, typename pos_t, bool PACKED, bool CONTIG = false, bool PAST_CACHE = false>
-__global__ __launch_bounds__(kWave * MAXW) __attribute__((amdgpu_num_sgpr(80)))
+__global__ __launch_bounds__(kWave * MAXW)
 __attribute__((amdgpu_waves_per_eu(PACKED && V * J <= 16 && !(CONTIG && V * J > 8) ? 8 : 1))) void fused_regs_kernel(
     const typename E::raw_t* __restrict__ x, typename E::raw_t* __restrict__ values,
     const IndexOut indices, const Geom g, uint32_t tiles, uint32_t split, uint32_t hand_off,
