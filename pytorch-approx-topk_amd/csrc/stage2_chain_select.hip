@@ -464,7 +464,11 @@ constexpr int kSoloWaves = kSoloThreads / select::kWave;
 constexpr uint32_t kSoloRankDirect = 512;
 static_assert((uint32_t)kSoloThreads == kSoloSegment, "a thread's u-th candidate lies in segment u");
 
-template <typename E, int NPT, bool OWN_RANGE, bool TIES = (sizeof(typename E::raw_t) == 1 || NPT <= 16)>
+// FULL: the row has exactly NPT * 1024 candidates, so that every key a thread holds exists and
+// nothing has to say which do (32 wave-wide masks otherwise, which the kernel with 32 keys per
+// thread has no scalar registers for).
+template <typename E, int NPT, bool OWN_RANGE, bool TIES = (sizeof(typename E::raw_t) == 1 || NPT <= 16),
+          bool FULL = false>
 __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
     const typename E::raw_t* __restrict__ cand_values, const int64_t* __restrict__ cand_indices, uint32_t k0,
     uint32_t k, uint32_t groups, int index_bits, const uint2* __restrict__ range, uint32_t entries,
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   // through every key of the row -- and short of registers: the keys alone take
   // up to 64 of its 128.)
   uint32_t key[NPT];
-  auto valid = [&](int u) -> bool { return (uint32_t)u * kSoloThreads + tid < k0; };
+  auto valid = [&](int u) -> bool { return FULL || (uint32_t)u * kSoloThreads + tid < k0; };
   {
     raw_t raw[NPT];
 #pragma unroll
@@ -589,7 +593,7 @@ __global__ __launch_bounds__(kSoloThreads) void chain_solo_kernel(
   // whole-row path below.
   const bool list_it = cut_digit && f.count <= kListCap;
   const uint32_t own = g * kSoloThreads + tid;  // this thread's candidate of segment g
-  const bool own_valid = own < k0;
+  const bool own_valid = FULL || own < k0;
   // survivors above the cut digit (or in it, when it belongs whole) in the
   // segments before this one, and the members of a cut digit: listed, or flagged for the
   // look at their indices below
@@ -934,7 +938,9 @@ int launch_chain_typed(const ChainPlan& pl, const void* cand_values, const int64
       raw_t* out = static_cast<raw_t*>(values);
 #define ATK_SOLO(NPT, OWN)                                                                                       \
   {                                                                                                              \
+    constexpr bool kTies = sizeof(raw_t) == 1 || NPT <= 16;                                                      \
     auto kern = chain_solo_kernel<E, NPT, OWN>;                                                                  \
+    if (k0 == (int64_t)NPT * kSoloThreads) kern = chain_solo_kernel<E, NPT, OWN, kTies, true>;                    \
     if (solo_lds > 48 * 1024 &&                                                                                  \
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,     \
                             (int)solo_lds) != hipSuccess)                                                        \
